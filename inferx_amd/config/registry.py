@@ -1,4 +1,4 @@
-"""One registry: architecture name (config.json `architectures[0]`) -> config class.
+"""One registry: architecture name (config.json `architectures[0]`, or `architecture`) -> config class.
 
 A config class has `from_dict(dict) -> config` and the config has
 `to_dict()`, `validate()` and `model_spec() -> ModelSpec`.  An unknown name is an
@@ -38,8 +38,11 @@ def config_class_for(name: str) -> Type:
 
 def config_from_dict(raw: Dict[str, Any]):
     archs = raw.get("architectures")
+    if archs is None and isinstance(raw.get("architecture"), str):  # some designs name themselves with one string
+        archs = [raw["architecture"]]
     if not isinstance(archs, list) or len(archs) != 1 or not isinstance(archs[0], str):
-        raise ConfigError("config.json: 'architectures' must be a list with exactly one name")
+        raise ConfigError("config.json: 'architectures' must be a list with exactly one name "
+                          "(or 'architecture' one name)")
     cfg = config_class_for(archs[0]).from_dict(raw)
     cfg.validate()
     return cfg

@@ -714,3 +714,141 @@ def measured_ceilings(device=None, read_bytes: int = 4 << 30) -> dict:
         stop.synchronize()
         best_mfma = max(best_mfma, flops.value / (start.elapsed_time(stop) * 1e-3) / 1e12)
     return {"hbm_read_gbs": round(best_read, 1), "mfma_bf16_tflops": round(best_mfma, 1)}
+
+
+# ---------------------------------------------------------------------------
+def _f32_vec(t: Optional[torch.Tensor], n: int, what: str):
+    if t is None:
+        return None
+    _need(t.dtype == torch.float32 and t.numel() == n, f"{what} must hold {n} float32 numbers")
+    return _ptr(t)
+
+
+class ShiftOperands:
+    """What a token shift needs of a step: the blend per channel (float32 [width]), the state [slots, width] and the
+    step's index arrays on the device."""
+
+    def __init__(self, mix, state, seq_of_token, q_start, state_slots, positions):
+        self.mix, self.state = mix, state
+        self.seq_of_token, self.q_start, self.state_slots, self.positions = seq_of_token, q_start, state_slots, positions
+
+    def check(self, tokens: int, width: int) -> None:
+        _need(self.mix.dtype == torch.float32 and self.mix.numel() == width, "the blend must be float32 [width]")
+        _need(self.state.dtype == torch.float32 and self.state.dim() == 2 and self.state.shape[1] == width
+              and self.state.is_contiguous(), "the state must be float32 [slots, width]")
+        _is_i32(self.seq_of_token, tokens)
+        _is_i32(self.positions, tokens)
+        _is_i32(self.q_start)
+        _is_i32(self.state_slots)
+        _need(self.q_start.numel() == self.state_slots.numel() + 1, "q_start must hold one entry more than there are requests")
+
+
+def add_dyt(h: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional[torch.Tensor], weight: torch.Tensor,
+            bias: Optional[torch.Tensor], alpha: float, out: torch.Tensor, rows: Optional[torch.Tensor] = None,
+            h_out: Optional[torch.Tensor] = None, shift: Optional[ShiftOperands] = None) -> None:
+    """out = tanh(alpha * v) * weight + bias with v = h + gain * delta, optionally blended with the row before
+    (`shift`).  v is written to `h_out` (h itself if not given) unless `rows` picks rows out; a shifted call needs
+    an `h_out` that is not h."""
+    H = h.shape[1]
+    _need(h.dtype == torch.float32 and h.dim() == 2, "the residual stream is float32 [T, width]")
+    _need(out.shape[1] == H, "width mismatch")
+    n_out = out.shape[0]
+    if rows is None:
+        _need(n_out == h.shape[0], "out must have a row per row of h")
+    else:
+        _is_i32(rows, n_out)
+    if delta is not None:
+        _need(delta.shape == h.shape, "delta must have the shape of h")
+    target = h if h_out is None else h_out
+    _need(target.dtype == torch.float32 and target.shape == h.shape, "h_out must be float32 of the shape of h")
+    if shift is not None:
+        _need(rows is None, "a shifted call takes all rows")
+        _need(target.data_ptr() != h.data_ptr(), "a shifted call cannot update the stream in place")
+        shift.check(h.shape[0], H)
+    write = delta is not None or target.data_ptr() != h.data_ptr()
+    s = shift
+    _call("ix_add_dyt", _ptr(h), _ptr(target) if (write and rows is None) else None, _ptr(delta),
+          _i32(_dt(delta) if delta is not None else F32), _f32_vec(gain, H, "the gain"), _f32_vec(weight, H, "the weight"),
+          _f32_vec(bias, H, "the bias"), _f32(alpha), _ptr(out), _i32(_dt(out)), _ptr(rows), _i64(n_out), _i64(H),
+          _ptr(s.mix) if s else None, _ptr(s.state) if s else None, _ptr(s.seq_of_token) if s else None,
+          _ptr(s.q_start) if s else None, _ptr(s.state_slots) if s else None, _ptr(s.positions) if s else None, _stream())
+
+
+def token_shift(x: torch.Tensor, out: torch.Tensor, shift: ShiftOperands) -> None:
+    """out[t] = x[t] + (x[t-1] - x[t]) * blend; the row before a request's first row comes from its state slot
+    (zero at position 0), which is left holding the request's last row."""
+    T, W = x.shape
+    _need(out.shape == x.shape and out.dtype == x.dtype and out.data_ptr() != x.data_ptr(), "out must be another tensor like x")
+    shift.check(T, W)
+    _call("ix_token_shift", _ptr(x), _ptr(out), _i32(_dt(x)), _ptr(shift.mix), _ptr(shift.state), _ptr(shift.seq_of_token),
+          _ptr(shift.q_start), _ptr(shift.state_slots), _ptr(shift.positions), _i64(T), _i64(W), _stream())
+
+
+def scale_columns(x: torch.Tensor, gain: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, i] = x[t, i] * gain[i]."""
+    T, W = x.shape
+    _need(out.shape == x.shape and out.dtype == x.dtype, "out must be like x")
+    _call("ix_scale_columns", _ptr(x), _ptr(out), _i32(_dt(x)), _f32_vec(gain, W, "the gain"), _i64(T), _i64(W), _stream())
+
+
+def _check_kv(q_dtype, k_cache, v_cache, kv_heads, head_dim, value_dim):
+    _need(k_cache.dtype == q_dtype and v_cache.dtype == q_dtype, "cache dtype differs from the activations'")
+    _need(k_cache.dim() == 4 and k_cache.shape[1] == kv_heads and k_cache.shape[3] == head_dim,
+          "key cache must be [pages, kv_heads, page_size, head_dim]")
+    _need(v_cache.shape == (k_cache.shape[0], kv_heads, value_dim, k_cache.shape[2]),
+          "value cache must be [pages, kv_heads, value_dim, page_size]")
+
+
+def qk_norm_append(qkv: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float,
+                   v_first: Optional[torch.Tensor], blend: float, v_out: Optional[torch.Tensor],
+                   slots: Optional[torch.Tensor], q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
+                   v_cache: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int, value_dim: int) -> None:
+    """After the q|k|v product (rows of `qkv`, which may be longer than the three): RMS norm over all of a token's
+    query numbers (`q_norm` float32 [heads * head_dim]) and over all of its key numbers, values blended with
+    `v_first` (v = (1 - blend) v + blend v_first), written to `v_out` if given, queries to `q_out`, keys and
+    values to the cache."""
+    T, stride = qkv.shape
+    qd, kd, vd = heads * head_dim, kv_heads * head_dim, kv_heads * value_dim
+    _need(stride >= qd + kd + vd and qkv.is_contiguous(), "a row of the product is shorter than q, k and v together")
+    _need(q_out.dtype == qkv.dtype and q_out.numel() == T * qd, "q_out mismatch")
+    for t in (v_first, v_out):
+        if t is not None:
+            _need(t.dtype == qkv.dtype and t.numel() == T * vd and t.is_contiguous(), "values of another layer mismatch")
+    page_size = 1
+    if slots is not None:
+        _need(k_cache is not None and v_cache is not None, "the cache is needed where slots are given")
+        _check_kv(qkv.dtype, k_cache, v_cache, kv_heads, head_dim, value_dim)
+        page_size = k_cache.shape[2]
+        _is_i32(slots, T)
+    _call("ix_qk_norm_append", _ptr(qkv), _i32(_dt(qkv)), _i64(stride), _f32_vec(q_norm, qd, "the query norm's weight"),
+          _f32_vec(k_norm, kd, "the key norm's weight"), _f32(eps), _ptr(v_first), _f32(blend), _ptr(v_out), _ptr(slots),
+          _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _i64(T), _i32(heads), _i32(kv_heads), _i32(head_dim),
+          _i32(value_dim), _i32(page_size), _stream())
+
+
+def attention_talk_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                         seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor,
+                         talk: Optional[torch.Tensor], sink: Optional[torch.Tensor], gate: Optional[torch.Tensor],
+                         scale: float, window: int = 0) -> None:
+    """Paged attention whose heads' scores are mixed before the softmax (`talk` float32 [heads, heads]), with a
+    sink per head in the softmax (`sink` float32 [heads]) and a sigmoid gate per head on the result (`gate`
+    [T, heads] in the activations' type, rows may be strided).  q [T, heads, head_dim], out [T, heads, value_dim]."""
+    T, heads, d = q.shape
+    kv_heads, vd = k_cache.shape[1], v_cache.shape[2]
+    _need(out.shape == (T, heads, vd) and out.dtype == q.dtype, "out must be [T, heads, value_dim]")
+    _check_kv(q.dtype, k_cache, v_cache, kv_heads, d, vd)
+    _need(block_table.dim() == 2, "block table must be [requests, pages]")
+    _is_i32(block_table)
+    _is_i32(seq_of_token, T)
+    _is_i32(positions, T)
+    gate_ptr, gate_stride = None, 0
+    if gate is not None:
+        _need(gate.dtype == q.dtype and gate.shape == (T, heads) and gate.stride(1) == 1 and gate.is_cuda,
+              "the gate must be [T, heads] in the activations' type")
+        gate_ptr, gate_stride = gate.data_ptr(), gate.stride(0)
+    _call("ix_attention_talk_plain", _ptr(q), _ptr(k_cache), _ptr(v_cache), _i32(_dt(q)), _ptr(block_table),
+          _ptr(seq_of_token), _ptr(positions), _ptr(out),
+          None if talk is None else _f32_vec(talk, heads * heads, "the mixing matrix"),
+          None if sink is None else _f32_vec(sink, heads, "the sinks"), gate_ptr, _i64(gate_stride), _i64(T),
+          _i32(heads), _i32(kv_heads), _i32(d), _i32(vd), _i32(k_cache.shape[2]), _i32(block_table.shape[1]),
+          _f32(scale), _i32(window), _stream())

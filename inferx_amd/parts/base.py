@@ -10,6 +10,8 @@ object, and does not know which model it is in.  Seven kinds:
   FeedForward       forward(ctx, x) -> delta          (dense or experts)
   Block             forward(ctx, h, pending, caches) -> pending delta; names the parts it arranges
   Head              forward(ctx, x) -> float32 logits [rows, vocab]
+  BranchGain        apply(delta) -> the delta with a learned gain per channel, applied where it is added
+  TokenShift        forward(ctx, x, cache) -> rows blended with the rows of the tokens before them
 
 Every part lists the tensors it needs (`param_specs`) under local names; the
 `PartSpec` maps those to checkpoint names.  `bind` receives the loaded tensors
@@ -30,12 +32,13 @@ from ..config.spec import PartSpec
 
 @dataclass(frozen=True)
 class ParamSpec:
-    """One tensor a part needs.  `init`: 'normal' (std = `std`), 'ones' or 'zeros'."""
+    """One tensor a part needs.  `init`: 'normal' (mean `mean`, standard deviation `std`), 'ones' or 'zeros'."""
 
     name: str
     shape: Tuple[int, ...]
     init: str = "normal"
     std: float = 0.02
+    mean: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -63,9 +66,11 @@ class CacheNeed:
     window: int = 0
 
     @staticmethod
-    def keys_and_values(kv_heads: int, head_dim: int, window: int = 0) -> "CacheNeed":
-        """Attention's cache: keys [pages, kv_heads, page_size, head_dim] and values transposed within a page."""
-        return CacheNeed((CacheArray("k", kv_heads, head_dim), CacheArray("v", kv_heads, head_dim, transposed=True)),
+    def keys_and_values(kv_heads: int, head_dim: int, window: int = 0, value_dim: Optional[int] = None) -> "CacheNeed":
+        """Attention's cache: keys [pages, kv_heads, page_size, head_dim] and values transposed within a page
+        (of `value_dim` numbers where they are not as wide as the keys)."""
+        return CacheNeed((CacheArray("k", kv_heads, head_dim),
+                          CacheArray("v", kv_heads, head_dim if value_dim is None else value_dim, transposed=True)),
                          window)
 
 
@@ -93,6 +98,20 @@ class LazyDelta:
     def add_rmsnorm(self, ctx, h, weight, eps, rows, out) -> bool:
         """h += delta; out = rmsnorm(h) * weight.  Returns False if this case is not fused (then nothing was done)."""
         return False
+
+
+class ScaledDelta(LazyDelta):
+    """A branch's result with a learned gain per channel that is not applied yet: delta[t, i] * gain[i] (gain
+    float32 [width]).  A norm that adds with a gain takes both as they are; any other consumer gets the product."""
+
+    def __init__(self, tensor, gain):
+        self.tensor, self.gain = tensor, gain
+
+    def materialize(self, ctx):
+        from .. import ops
+        out = ctx.rt.empty(tuple(self.tensor.shape), self.tensor.dtype)
+        ops.scale_columns(self.tensor, self.gain, out)
+        return out
 
 
 def resolve_delta(ctx, delta):
@@ -156,12 +175,22 @@ class Part:
 
 
 class Norm(Part):
+    # True: `forward` takes `h_in`, a buffer to read the stream from while the sum is written to h
+    reads_stream_elsewhere = False
+
     def rms_operands(self):
         """(weight, eps) if this is a plain RMS norm that another kernel may apply, else None."""
         return None
 
     def forward(self, ctx, h, delta=None, rows=None):
         raise NotImplementedError
+
+    def forward_shifted(self, ctx, h, delta, shift, cache):
+        """The normalised rows of h + delta with `shift` (a `TokenShift`, whose state is `cache`) applied to them:
+        (rows, moved).  `moved` is None if h was updated in place; a norm that shifts in its own kernel cannot do
+        that (a row's result reads the row before it) and returns the updated stream as `moved`, a buffer of its
+        own, leaving h as it was: the caller goes on from `moved`."""
+        return shift.forward(ctx, self.forward(ctx, h, delta), cache), None
 
 
 class PositionEncoding(Part):
@@ -195,6 +224,22 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class BranchGain(Part):
+    """A learned gain per channel on a branch's result (a mixer's or a feed-forward's) before it is added to the
+    residual stream."""
+
+    def apply(self, delta):
+        raise NotImplementedError
+
+
+class TokenShift(Part):
+    """Blends every row with the row of the token before it in the same sequence; the last row of a step is kept
+    per request for the next step (`state_need`)."""
+
+    def forward(self, ctx, x, cache):
+        raise NotImplementedError
+
+
 class Block:
     """An arrangement of parts around the residual stream.  `part_kinds` names the parts the arrangement needs
     and the kind of each (a key of the registries); names in `optional_parts` may be left out of a `LayerSpec`.
@@ -216,11 +261,12 @@ class Block:
 
 _REGISTRIES: Dict[str, Dict[str, Callable[..., Any]]] = {
     "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {}, "head": {},
+    "gain": {}, "shift": {},
 }
 
 
 def register_part(kind: str, name: str, factory: Callable[..., Any]) -> None:
-    """kind: 'norm' | 'position' | 'mixer' | 'feed_forward' | 'block' | 'embedding' | 'head'.  A block is
+    """kind: 'norm' | 'position' | 'mixer' | 'feed_forward' | 'block' | 'embedding' | 'head' | 'gain' | 'shift'.  A block is
     registered by its class (see `Block`), every other kind by a callable that takes the `PartSpec`'s parameters."""
     if kind not in _REGISTRIES:
         raise KeyError(f"no such kind of part: {kind!r} (known: {', '.join(_REGISTRIES)})")

@@ -9,7 +9,7 @@ says so gets norm2 unapplied (`LazyNorm`) and applies it in its first kernel.
 """
 from __future__ import annotations
 
-from .base import Block, LazyNorm, register_part
+from .base import Block, LazyNorm, register_part, resolve_delta
 
 
 class PreNormBlock(Block):
@@ -24,4 +24,51 @@ class PreNormBlock(Block):
         return self.feed_forward.forward(ctx, self.feed_forward_norm.forward(ctx, h, a))
 
 
+class GainedPreNormBlock(Block):
+    """`prenorm` with three optional additions, each a part of its own:
+
+        x = shift(norm1(h + pending));  h += gain1 * mixer(x);  pending = gain2 * feed_forward(norm2(h))
+
+    `mixer_gain` / `feed_forward_gain` (kind "gain"): a learned gain per channel on the branch's result;
+    `mixer_shift` (kind "shift"): the mixer reads rows blended with the rows of the tokens before them.  The
+    feed-forward and its norm may be left out; the mixer's delta then stays pending for the next layer."""
+
+    graph_safe = True
+    part_kinds = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm", "feed_forward_norm": "norm",
+                  "mixer_gain": "gain", "feed_forward_gain": "gain", "mixer_shift": "shift"}
+    optional_parts = ("feed_forward", "feed_forward_norm", "mixer_gain", "feed_forward_gain", "mixer_shift")
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        if (self.feed_forward is None) != (self.feed_forward_norm is None):
+            raise KeyError("a feed-forward and the norm before it come together or not at all")
+
+    def forward(self, ctx, h, pending, caches):
+        moved = None
+        if self.mixer_shift is not None:
+            # a norm that shifts in its own kernel leaves the updated stream in a buffer of its own (`moved`)
+            x, moved = self.mixer_norm.forward_shifted(ctx, h, pending, self.mixer_shift, caches.get("mixer_shift"))
+        else:
+            x = self.mixer_norm.forward(ctx, h, pending)
+        a = self.mixer.forward(ctx, x, caches.get("mixer"))
+        if self.mixer_gain is not None:
+            a = self.mixer_gain.apply(resolve_delta(ctx, a))
+        if self.feed_forward is None:
+            if moved is not None:
+                h.copy_(moved)
+            return a
+        if moved is not None and self.feed_forward_norm.reads_stream_elsewhere:
+            # the next norm reads the stream where it is now and writes it back to h
+            x = self.feed_forward_norm.forward(ctx, h, a, h_in=moved)
+        else:
+            if moved is not None:
+                h.copy_(moved)
+            x = self.feed_forward_norm.forward(ctx, h, a)
+        f = self.feed_forward.forward(ctx, x)
+        if self.feed_forward_gain is not None:
+            f = self.feed_forward_gain.apply(resolve_delta(ctx, f))
+        return f
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "prenorm_gained", GainedPreNormBlock)

@@ -92,6 +92,8 @@ def random_tensors(model, seed: int, dtype: str = "bfloat16", device: str = "cpu
             t = torch.zeros(p.shape, dtype=torch.float32, device=device)
         elif p.init == "normal":
             t = counter_normal(seed, name, p.shape, p.std, device)
+            if getattr(p, "mean", 0.0):
+                t = t + float(p.mean)
         else:
             raise ValueError(f"tensor {name!r}: unknown init {p.init!r}")
         out[name] = t.to(store)
