@@ -852,3 +852,48 @@ def attention_talk_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
           None if sink is None else _f32_vec(sink, heads, "the sinks"), gate_ptr, _i64(gate_stride), _i64(T),
           _i32(heads), _i32(kv_heads), _i32(d), _i32(vd), _i32(k_cache.shape[2]), _i32(block_table.shape[1]),
           _f32(scale), _i32(window), _stream())
+
+
+def attention_talk_mfma_heads_per_wave(heads: int, kv_heads: int, head_dim: int, value_dim: int, page_size: int) -> int:
+    """How many heads a wavefront of `attention_talk_mfma` takes for these sizes; 0 if the kernel does not take them."""
+    fn = _functions.get("ix_attention_talk_mfma_heads_per_wave")
+    if fn is None:
+        fn = _functions["ix_attention_talk_mfma_heads_per_wave"] = lib().ix_attention_talk_mfma_heads_per_wave
+    return int(fn(heads, kv_heads, head_dim, value_dim, page_size))
+
+
+def attention_talk_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                        tiles: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, n_splits: int,
+                        workspace: Optional[torch.Tensor], talk: Optional[torch.Tensor], sink: Optional[torch.Tensor],
+                        gate: Optional[torch.Tensor], scale: float) -> None:
+    """`attention_talk_plain` on the matrix cores (bfloat16, no window).  `tiles` int32 [3, n_tiles]: request, first
+    row and rows (at most 16) of each query tile; the keys of a tile are cut into `n_splits` slices, whose parts go
+    through `workspace` (float32, T * heads * n_splits * (value_dim + 2) entries) when there are several."""
+    T, heads, d = q.shape
+    _need(q.dtype == torch.bfloat16, "the matrix-core attention kernel is bfloat16 only")
+    kv_heads, vd = k_cache.shape[1], v_cache.shape[2]
+    _need(out.shape == (T, heads, vd) and out.dtype == q.dtype, "out must be [T, heads, value_dim]")
+    _check_kv(q.dtype, k_cache, v_cache, kv_heads, d, vd)
+    _need(block_table.dim() == 2, "block table must be [requests, pages]")
+    _is_i32(block_table)
+    _is_i32(positions, T)
+    _is_i32(tiles)
+    _need(tiles.dim() == 2 and tiles.shape[0] == 3 and tiles.is_contiguous(), "tiles must be int32 [3, n_tiles]")
+    part_o = part_ml = None
+    if n_splits > 1:
+        need = T * heads * n_splits * (vd + 2)
+        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need,
+              f"workspace of {need} float32 needed")
+        part_o = workspace
+        part_ml = workspace[T * heads * n_splits * vd:]
+    gate_ptr, gate_stride = None, 0
+    if gate is not None:
+        _need(gate.dtype == q.dtype and gate.shape == (T, heads) and gate.stride(1) == 1 and gate.is_cuda,
+              "the gate must be [T, heads] in the activations' type")
+        gate_ptr, gate_stride = gate.data_ptr(), gate.stride(0)
+    _call("ix_attention_talk_mfma", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]),
+          _ptr(tiles[1]), _ptr(tiles[2]), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml),
+          None if talk is None else _f32_vec(talk, heads * heads, "the mixing matrix"),
+          None if sink is None else _f32_vec(sink, heads, "the sinks"), gate_ptr, _i64(gate_stride), _i64(T),
+          _i32(tiles.shape[1]), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(vd), _i32(k_cache.shape[2]),
+          _i32(block_table.shape[1]), _f32(scale), _stream())

@@ -22,6 +22,7 @@ from typing import List, Optional
 import torch
 
 from .. import ops
+from .attention import QUERY_TILE, _n_splits, plan_tiles
 from .base import CacheNeed, Mixer, ParamSpec, register_part
 from .dense_mlp import stack_rows
 
@@ -135,9 +136,35 @@ class TalkingAttention(Mixer):
         self.attend(ctx, q, cache, gate, out)
         return rt.linear(out.view(T, self.out_dim), self.w_out)
 
+    def capture_plan(self, ctx, requests: int, longest: int) -> None:
+        """The query tiles of a step of one token per request never change: tile i = request i, row i, one query
+        (the plan that `plan_tiles` would make from the host's arrays)."""
+        key = ("attention_tiles_host", QUERY_TILE)
+        if key not in ctx.memo:
+            tiles = torch.tensor([list(range(requests)), list(range(requests)), [1] * requests], dtype=torch.int32,
+                                 device=ctx.rt.device)
+            ctx.memo[key] = (tiles, requests, longest)
+
     def attend(self, ctx, q, cache, gate, out) -> None:
-        ops.attention_talk_plain(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.seq_of_token, ctx.positions,
-                                 out, self.talk, self.sink, gate, self.scale, self.window)
+        """bfloat16 with heads, values and pages in multiples of 16 and no window: the matrix-core kernel, a workgroup
+        per tile of sixteen queries and slice of keys; else the plain one."""
+        page_size = cache.k.shape[2]
+        table = ctx.block_tables[cache.group]
+        per_wave = 0
+        if q.dtype == torch.bfloat16 and self.window == 0:
+            per_wave = ops.attention_talk_mfma_heads_per_wave(self.num_heads, self.num_kv_heads, self.head_dim,
+                                                              self.value_dim, page_size)
+        if per_wave == 0:
+            ops.attention_talk_plain(q, cache.k, cache.v, table, ctx.seq_of_token, ctx.positions, out, self.talk,
+                                     self.sink, gate, self.scale, self.window)
+            return
+        tiles, n_tiles, longest = plan_tiles(ctx, QUERY_TILE)
+        n_splits = _n_splits(n_tiles * (self.num_heads // per_wave), longest, 0, QUERY_TILE)
+        work = None
+        if n_splits > 1:
+            work = ctx.rt.empty((q.shape[0] * self.num_heads * n_splits * (self.value_dim + 2),), torch.float32)
+        ops.attention_talk_mfma(q, cache.k, cache.v, table, tiles, ctx.positions, out, n_splits, work, self.talk,
+                                self.sink, gate, self.scale)
 
 
 register_part("mixer", "talking_attention", TalkingAttention)
