@@ -28,6 +28,12 @@ function:
 
     python bench.py --workload portion --shape a27b|57b --prefill-tokens N --prefill-context C [--layers L]
 
+and the Pelalix design (Dynamic Tanh norms, token shift, attention whose heads' scores are mixed, with sinks and gates)
+beside the dense layers of the Qwen2-MoE architecture at equal sizes (the same width, heads, key/value heads, head size,
+feed-forward width, vocabulary and layers), both through the step function, at a few sizes of real models' layers:
+
+    python bench.py --workload pelalix [--sizes 2k,4k] [--layers L] [--batch B] [--prompt-len C] [--prefill-tokens N]
+
 and a whole batch through the engine's loop (scheduler, portions, decode graphs as they come, sampling) at the same
 shape:
 
@@ -406,6 +412,133 @@ def run_offline(args) -> int:
     return 0
 
 
+# Layer sizes for `--workload pelalix`: width, heads, key/value heads, head size, feed-forward width, vocabulary
+PELALIX_SIZES = {
+    "1k": dict(width=1024, heads=8, kv_heads=2, dim=128, ff=2816, vocab=32000),
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=5632, vocab=32000),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=11008, vocab=32000),
+}
+
+
+class _SpecOnly:
+    """A configuration that is nothing but a `ModelSpec` (what the runner reads of a configuration)."""
+
+    eos_token_ids = ()
+
+    def __init__(self, spec):
+        self._spec = spec
+
+    def model_spec(self):
+        return self._spec
+
+
+def run_pelalix(args) -> int:
+    """Prefill of one prompt and decode steps of a batch, through the step function, for the Pelalix design and for
+    the Qwen2-MoE architecture's dense layers (attention with rotation, RMS norms, the same gated feed-forward) at
+    equal sizes.  One JSON line; per size and model: milliseconds and tokens a second of both phases, the matrix
+    flops and the bytes of a decode step against the published peaks, and Pelalix's time over the other's."""
+    import dataclasses
+
+    import torch
+    from inferx_amd.config import ScheduleEntry, config_from_dict
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_model
+    from inferx_amd.weights import random_tensors
+
+    L = args.layers or 4
+    B, C, N = args.batch, args.prompt_len, args.prefill_tokens
+    rt = Runtime(args.dtype, "cuda:0")
+    elt = 2 if args.dtype == "bfloat16" else 4
+    peak = PEAK_TFLOPS["bf16" if elt == 2 else "fp32"] * 1e12
+    gen = torch.Generator().manual_seed(1234)
+    out = {}
+
+    def specs(z):
+        pel = {"architecture": "Pelalix", "vocab": z["vocab"], "width": z["width"], "embedding": {"scale": 1.0},
+               "norm": {"eps": 1e-6},
+               "layers": [{"type": "attention",
+                           "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                                     "scale": z["dim"] ** -0.5, "v_mix": True},
+                           "mlp": {"kind": "dense", "ff": z["ff"]}} for _ in range(L)]}
+        # the other architecture wants one layer of experts: it is configured last and left out of the model
+        qwen = {"architectures": ["Qwen2MoeForCausalLM"], "num_hidden_layers": L + 1, "hidden_size": z["width"],
+                "num_attention_heads": z["heads"], "num_key_value_heads": z["kv_heads"], "head_dim": z["dim"],
+                "num_experts": 2, "num_experts_per_tok": 1, "moe_intermediate_size": 64,
+                "shared_expert_intermediate_size": 0, "intermediate_size": z["ff"], "mlp_only_layers": list(range(L)),
+                "vocab_size": z["vocab"], "rope_theta": 1e6, "rms_norm_eps": 1e-6, "max_position_embeddings": 0}
+        spec = config_from_dict(qwen).model_spec()
+        dense = dataclasses.replace(spec, layers=spec.layers[:L], schedule=[ScheduleEntry(i) for i in range(L)])
+        return {"pelalix": config_from_dict(pel).model_spec(), "qwen2_dense": dense}
+
+    def measure(spec, z):
+        model = build_model(spec)
+        weights = {k: rt.place(v) for k, v in random_tensors(model, seed=0, dtype=args.dtype, device="cuda:0").items()}
+        cap = -(-(max(C + args.warmup + args.steps + 8, N) + 16) // PAGE) * PAGE
+        runner = ModelRunner(_SpecOnly(spec), weights, rt, page_size=PAGE, num_pages=(B + 1) * cap // PAGE,
+                             max_requests=B + 1, max_seq_len=cap, model=model)
+        runner.capture_after = 1
+        toks = lambda n: torch.randint(0, z["vocab"], (n,), generator=gen).tolist()
+        times = []
+        for _ in range(4):  # the prompt of N tokens in one step
+            runner.add_request("p")
+            prompt = toks(N)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            runner.run_entries([("p", prompt, [N - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            runner.end_request("p")
+        pre = min(times[1:])
+        for r in range(B):  # B requests with C tokens behind them, then steps of one token each
+            runner.add_request(r)
+            for at in range(0, C, 2048):
+                runner.run_entries([(r, toks(min(2048, C - at)), [])])
+        step = lambda: runner.run_entries([(r, toks(1), [0]) for r in range(B)])
+        for _ in range(max(args.warmup, 2)):
+            step()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        dec = (time.perf_counter() - t) / args.steps
+        for r in range(B):
+            runner.end_request(r)
+        W, H, G, d, ff, V = z["width"], z["heads"], z["kv_heads"], z["dim"], z["ff"], z["vocab"]
+        per_token = W * (H * d + 2 * G * d) + H * d * W + 3 * W * ff
+        flops = 2.0 * N * L * per_token + 2.0 * V * W + L * 2.0 * 2.0 * H * d * N * (N + 1) / 2.0
+        bytes_dec = (L * per_token + V * W + L * 2 * G * d * (C + args.warmup + args.steps // 2) * B) * elt
+        del runner, weights, model
+        torch.cuda.empty_cache()
+        return {"prefill_ms": round(pre * 1e3, 3), "prefill_tokens_s": round(N / pre, 1),
+                "prefill_tflops": round(flops / pre / 1e12, 1), "prefill_frac_of_peak": round(flops / pre / peak, 4),
+                "decode_ms": round(dec * 1e3, 3), "decode_tokens_s": round(B / dec, 1),
+                "decode_gbs": round(bytes_dec / dec / 1e9, 1), "decode_frac_of_peak": round(bytes_dec / dec / 1e9 / PEAK_HBM_GBS, 4)}
+
+    for name in [n for n in args.sizes.split(",") if n]:
+        z = PELALIX_SIZES[name]
+        res = {}
+        for which, spec in specs(z).items():
+            log(f"{name}: {which}")
+            res[which] = measure(spec, z)
+            log(f"{name}: {which}: {res[which]}")
+        res["pelalix_over_qwen2_dense"] = {
+            "prefill": round(res["pelalix"]["prefill_ms"] / res["qwen2_dense"]["prefill_ms"], 3),
+            "decode": round(res["pelalix"]["decode_ms"] / res["qwen2_dense"]["decode_ms"], 3)}
+        out[name] = dict(res, sizes=z)
+    first = out[next(iter(out))]
+    print(json.dumps({
+        "metric": f"Pelalix decode tok/s @ batch {B} ({C}-token contexts), first size", "value": first["pelalix"]["decode_tokens_s"],
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["pelalix"]["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if elt == 2 else "fp32", "data": "synthetic: seeded random weights and token ids",
+        "config": {"model": "Pelalix beside Qwen2 dense layers at equal sizes", "layers": L, "global_batch": B,
+                   "seq_len": C, "prefill_tokens": N, "parallelism": "single GPU", "page_size": PAGE},
+        "sizes": out}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -415,7 +548,7 @@ def main() -> int:
                     help="fewer layers than the configuration has (sizes of a layer are never reduced)")
     ap.add_argument("--scarce", action="store_true", help="offline: so few pages that sequences are preempted")
     ap.add_argument("--workload", default="decode",
-                    choices=["decode", "mixed", "long", "mixed-small", "offline", "portion"],
+                    choices=["decode", "mixed", "long", "mixed-small", "offline", "portion", "pelalix"],
                     help="decode, mixed-small: the Qwen1.5-MoE-A2.7B shape (decode is the default); mixed, long: the "
                          "Qwen2-57B-A14B shape")
     ap.add_argument("--batch", type=int, default=8)
@@ -427,6 +560,7 @@ def main() -> int:
     ap.add_argument("--prefill-context", type=int, default=0,
                     help="portion: tokens that the request has read before the timed portion")
     ap.add_argument("--shape", default="a27b", choices=["a27b", "57b"], help="portion: whose layer sizes")
+    ap.add_argument("--sizes", default="2k,4k", help="pelalix: which of the layer sizes " + ", ".join(PELALIX_SIZES))
     ap.add_argument("--prompt-len", type=int, default=PROMPT,
                     help="tokens of every request's prompt before it decodes (the context of the decode steps)")
     args = ap.parse_args()
@@ -434,13 +568,15 @@ def main() -> int:
         print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
         return 2
     if args.steps is None:
-        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24, "offline": 0, "portion": 2}[args.workload]
+        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24, "offline": 0, "portion": 2, "pelalix": 32}[args.workload]
     if args.warmup is None:
-        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4, "offline": 0, "portion": 1}[args.workload]
+        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4, "offline": 0, "portion": 1, "pelalix": 4}[args.workload]
     if args.workload == "offline":
         return run_offline(args)
     if args.workload == "portion":
         return run_portion(args)
+    if args.workload == "pelalix":
+        return run_pelalix(args)
     if args.workload != "decode":
         return run_57b(args)
     if args.layers is None:
