@@ -14,7 +14,8 @@
 // ---------------------------------------------------------------------------
 // After the product: RMS norm over ALL of a token's query numbers at once (and over all of its key numbers),
 // the values blended with the values that an earlier layer made for the same token, queries out, keys and
-// values into the cache.  One workgroup per token.
+// values into the cache.  Three workgroups per token (blockIdx.y: queries, keys, values), so that what each has to
+// wait for -- its own numbers, their sum of squares, the weights -- runs side by side.
 template <typename T>
 __global__ void __launch_bounds__(256)
 qk_norm_append_kernel(const T* __restrict__ qkv, int64_t stride, const float* __restrict__ q_norm,
@@ -24,41 +25,42 @@ qk_norm_append_kernel(const T* __restrict__ qkv, int64_t stride, const float* __
                       int value_dim, int page_size) {
   __shared__ float red[16];
   const int64_t t = blockIdx.x;
+  const int part = blockIdx.y;
   const int q_dim = heads * head_dim, k_dim = kv_heads * head_dim, v_dim = kv_heads * value_dim;
   const T* row = qkv + t * stride;
-  float q_inv = 1.f, k_inv = 1.f;
-  if (q_norm) {
-    float sq = 0.f;
-    for (int i = threadIdx.x; i < q_dim; i += blockDim.x) {
-      const float v = ix_load(row + i);
-      sq += v * v;
-    }
-    q_inv = 1.0f / sqrtf(ix_block_sum(sq, red) / static_cast<float>(q_dim) + eps);
-  }
-  if (k_norm) {
-    float sq = 0.f;
-    for (int i = threadIdx.x; i < k_dim; i += blockDim.x) {
-      const float v = ix_load(row + q_dim + i);
-      sq += v * v;
-    }
-    k_inv = 1.0f / sqrtf(ix_block_sum(sq, red) / static_cast<float>(k_dim) + eps);
-  }
-  for (int i = threadIdx.x; i < q_dim; i += blockDim.x)
-    ix_store(q_out + t * q_dim + i, ix_load(row + i) * q_inv * (q_norm ? q_norm[i] : 1.f));
-  if (!slots) return;
-  const int64_t slot = slots[t];
+  if (part > 0 && !slots) return;
+  const int64_t slot = slots ? slots[t] : 0;
   const int64_t page = slot / page_size, off = slot % page_size;
-  for (int i = threadIdx.x; i < k_dim; i += blockDim.x) {
-    const int c = i / head_dim, e = i - c * head_dim;
-    ix_store(k_cache + ((page * kv_heads + c) * page_size + off) * head_dim + e,
-             ix_load(row + q_dim + i) * k_inv * (k_norm ? k_norm[i] : 1.f));
+  if (part == 2) {
+    for (int i = threadIdx.x; i < v_dim; i += blockDim.x) {
+      const int c = i / value_dim, e = i - c * value_dim;
+      float v = ix_load(row + q_dim + k_dim + i);
+      if (v_first) v = (1.0f - lambda) * v + lambda * ix_load(v_first + t * v_dim + i);
+      if (v_out) ix_store(v_out + t * v_dim + i, v);
+      ix_store(v_cache + ((page * kv_heads + c) * value_dim + e) * page_size + off, v);
+    }
+    return;
   }
-  for (int i = threadIdx.x; i < v_dim; i += blockDim.x) {
-    const int c = i / value_dim, e = i - c * value_dim;
-    float v = ix_load(row + q_dim + k_dim + i);
-    if (v_first) v = (1.0f - lambda) * v + lambda * ix_load(v_first + t * v_dim + i);
-    if (v_out) ix_store(v_out + t * v_dim + i, v);
-    ix_store(v_cache + ((page * kv_heads + c) * value_dim + e) * page_size + off, v);
+  const T* src = part == 0 ? row : row + q_dim;
+  const float* weight = part == 0 ? q_norm : k_norm;
+  const int n = part == 0 ? q_dim : k_dim;
+  float inv = 1.f;
+  if (weight) {
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      const float v = ix_load(src + i);
+      sq += v * v;
+    }
+    inv = 1.0f / sqrtf(ix_block_sum(sq, red) / static_cast<float>(n) + eps);
+  }
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = ix_load(src + i) * inv * (weight ? weight[i] : 1.f);
+    if (part == 0) {
+      ix_store(q_out + t * q_dim + i, v);
+    } else {
+      const int c = i / head_dim, e = i - c * head_dim;
+      ix_store(k_cache + ((page * kv_heads + c) * page_size + off) * head_dim + e, v);
+    }
   }
 }
 
@@ -72,7 +74,7 @@ extern "C" int ix_qk_norm_append(const void* qkv, int dtype, int64_t stride, con
              "a row of the product is shorter than q, k and v together");
   IX_REQUIRE(!slots || (k_cache && v_cache), "the cache is needed where slots are given");
   if (tokens == 0) return 0;
-  dim3 grid(tokens), block(256);
+  dim3 grid(tokens, 3), block(256);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(qk_norm_append_kernel<float>, grid, block, 0, stream, (const float*)qkv, stride, q_norm, k_norm,
                        eps, (const float*)v_first, lambda, (float*)v_out, slots, (float*)q_out, (float*)k_cache,

@@ -79,6 +79,89 @@ add_dyt_kernel(DytArgs a, TO* __restrict__ out, int64_t width) {
   }
 }
 
+// bfloat16 delta and result with a width that is a multiple of 4: four columns per thread, 16-byte accesses to
+// the stream, 8-byte ones to delta and result
+struct Four {
+  float v[4];
+};
+__device__ __forceinline__ Four dyt_sum4(const DytArgs& a, int64_t row, int64_t width, int64_t c, const Four& gain) {
+  const float4 h = *reinterpret_cast<const float4*>(a.h_in + row * width + c);
+  Four out{{h.x, h.y, h.z, h.w}};
+  if (a.delta) {
+    const uint2 d = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.delta) + row * width + c);
+    out.v[0] += gain.v[0] * __uint_as_float(d.x << 16);
+    out.v[1] += gain.v[1] * __uint_as_float(d.x & 0xffff0000u);
+    out.v[2] += gain.v[2] * __uint_as_float(d.y << 16);
+    out.v[3] += gain.v[3] * __uint_as_float(d.y & 0xffff0000u);
+  }
+  return out;
+}
+
+__global__ void __launch_bounds__(256)
+add_dyt_vec4_kernel(DytArgs a, uint16_t* __restrict__ out, int64_t width) {
+  const int64_t r = blockIdx.x;
+  const int64_t row = a.rows ? a.rows[r] : r;
+  int64_t prev_row = -1, last_row = -1, slot = 0;
+  bool first = false, from_state = false;
+  if (a.mix) {
+    const int64_t s = a.seq_of_token[row];
+    first = row == a.q_start[s];
+    if (first) {
+      from_state = a.positions[row] > 0;
+      last_row = a.q_start[s + 1] - 1;
+      slot = a.state_slots[s];
+    } else {
+      prev_row = row - 1;
+    }
+  }
+  for (int64_t c = 4 * (static_cast<int64_t>(blockIdx.y) * blockDim.x + threadIdx.x); c < width;
+       c += 4 * static_cast<int64_t>(gridDim.y) * blockDim.x) {
+    Four gain{{1.f, 1.f, 1.f, 1.f}}, b{{0.f, 0.f, 0.f, 0.f}}, w, n;
+    const float4 w4 = *reinterpret_cast<const float4*>(a.w + c);
+    w = Four{{w4.x, w4.y, w4.z, w4.w}};
+    if (a.gain) {
+      const float4 g4 = *reinterpret_cast<const float4*>(a.gain + c);
+      gain = Four{{g4.x, g4.y, g4.z, g4.w}};
+    }
+    if (a.b) {
+      const float4 b4 = *reinterpret_cast<const float4*>(a.b + c);
+      b = Four{{b4.x, b4.y, b4.z, b4.w}};
+    }
+    const Four v = dyt_sum4(a, row, width, c, gain);
+    if (a.h_out && !a.rows) *reinterpret_cast<float4*>(a.h_out + row * width + c) = make_float4(v.v[0], v.v[1], v.v[2], v.v[3]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) n.v[i] = tanhf(a.alpha * v.v[i]) * w.v[i] + b.v[i];
+    if (a.mix) {
+      Four before{{0.f, 0.f, 0.f, 0.f}};
+      if (first) {
+        if (from_state) {
+          const float4 s4 = *reinterpret_cast<const float4*>(a.state + slot * width + c);
+          before = Four{{s4.x, s4.y, s4.z, s4.w}};
+        }
+        Four n_last = n;
+        if (last_row != row) {
+          const Four vl = dyt_sum4(a, last_row, width, c, gain);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) n_last.v[i] = tanhf(a.alpha * vl.v[i]) * w.v[i] + b.v[i];
+        }
+        *reinterpret_cast<float4*>(a.state + slot * width + c) = make_float4(n_last.v[0], n_last.v[1], n_last.v[2], n_last.v[3]);
+      } else {
+        const Four vp = dyt_sum4(a, prev_row, width, c, gain);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) before.v[i] = tanhf(a.alpha * vp.v[i]) * w.v[i] + b.v[i];
+      }
+      const float4 m4 = *reinterpret_cast<const float4*>(a.mix + c);
+      const float m[4] = {m4.x, m4.y, m4.z, m4.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) n.v[i] += (before.v[i] - n.v[i]) * m[i];
+    }
+    uint2 o;
+    o.x = ix_f32_to_bf16(n.v[0]) | static_cast<uint32_t>(ix_f32_to_bf16(n.v[1])) << 16;
+    o.y = ix_f32_to_bf16(n.v[2]) | static_cast<uint32_t>(ix_f32_to_bf16(n.v[3])) << 16;
+    *reinterpret_cast<uint2*>(out + r * width + c) = o;
+  }
+}
+
 extern "C" int ix_add_dyt(const float* h_in, float* h_out, const void* delta, int delta_dtype, const float* gain,
                           const float* w, const float* b, float alpha, void* out, int out_dtype, const int32_t* rows,
                           int64_t n_out_rows, int64_t width, const float* mix, float* state,
@@ -96,6 +179,13 @@ extern "C" int ix_add_dyt(const float* h_in, float* h_out, const void* delta, in
   dim3 grid(n_out_rows, chunks), block(threads);
 #define LAUNCH(TD, TO) hipLaunchKernelGGL((add_dyt_kernel<TD, TO>), grid, block, 0, stream, a, (TO*)out, width)
   const int dd = delta ? delta_dtype : IX_F32;
+  auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (out_dtype == IX_BF16 && (!delta || delta_dtype == IX_BF16) && width % 4 == 0 && aligned(h_in) && aligned(h_out) &&
+      aligned(delta) && aligned(out) && aligned(gain) && aligned(w) && aligned(b) && aligned(mix) && aligned(state)) {
+    const int chunks4 = static_cast<int>(std::min<int64_t>((width / 4 + threads - 1) / threads, 64));
+    hipLaunchKernelGGL(add_dyt_vec4_kernel, dim3(n_out_rows, chunks4), block, 0, stream, a, (uint16_t*)out, width);
+    return ix_check_launch("ix_add_dyt");
+  }
   if (dd == IX_F32 && out_dtype == IX_F32) LAUNCH(float, float);
   else if (dd == IX_F32 && out_dtype == IX_BF16) LAUNCH(float, bf16_t);
   else if (dd == IX_BF16 && out_dtype == IX_F32) LAUNCH(bf16_t, float);

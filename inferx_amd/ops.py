@@ -865,7 +865,7 @@ def attention_talk_mfma_heads_per_wave(heads: int, kv_heads: int, head_dim: int,
 def attention_talk_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                         tiles: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, n_splits: int,
                         workspace: Optional[torch.Tensor], talk: Optional[torch.Tensor], sink: Optional[torch.Tensor],
-                        gate: Optional[torch.Tensor], scale: float) -> None:
+                        gate: Optional[torch.Tensor], scale: float, heads_per_wave: int = 0) -> None:
     """`attention_talk_plain` on the matrix cores (bfloat16, no window).  `tiles` int32 [3, n_tiles]: request, first
     row and rows (at most 16) of each query tile; the keys of a tile are cut into `n_splits` slices, whose parts go
     through `workspace` (float32, T * heads * n_splits * (value_dim + 2) entries) when there are several."""
@@ -896,4 +896,4 @@ def attention_talk_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
           None if talk is None else _f32_vec(talk, heads * heads, "the mixing matrix"),
           None if sink is None else _f32_vec(sink, heads, "the sinks"), gate_ptr, _i64(gate_stride), _i64(T),
           _i32(tiles.shape[1]), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(vd), _i32(k_cache.shape[2]),
-          _i32(block_table.shape[1]), _f32(scale), _stream())
+          _i32(block_table.shape[1]), _f32(scale), _i32(heads_per_wave), _stream())

@@ -22,7 +22,7 @@ from typing import List, Optional
 import torch
 
 from .. import ops
-from .attention import QUERY_TILE, _n_splits, plan_tiles
+from .attention import QUERY_TILE, plan_tiles
 from .base import CacheNeed, Mixer, ParamSpec, register_part
 from .dense_mlp import stack_rows
 
@@ -159,12 +159,28 @@ class TalkingAttention(Mixer):
                                      self.sink, gate, self.scale, self.window)
             return
         tiles, n_tiles, longest = plan_tiles(ctx, QUERY_TILE)
-        n_splits = _n_splits(n_tiles * (self.num_heads // per_wave), longest, 0, QUERY_TILE)
+        n_splits = key_slices(n_tiles, longest, ctx.one_token_each)
         work = None
         if n_splits > 1:
             work = ctx.rt.empty((q.shape[0] * self.num_heads * n_splits * (self.value_dim + 2),), torch.float32)
         ops.attention_talk_mfma(q, cache.k, cache.v, table, tiles, ctx.positions, out, n_splits, work, self.talk,
                                 self.sink, gate, self.scale)
+
+
+WORKGROUPS_WANTED = 512  # two per compute unit: the tiles of a causal triangle end at very different times
+MIN_KEYS_PER_SLICE = 128  # (a step of one token per request: a few rounds of the kernel)
+MIN_KEYS_PER_SLICE_OF_PORTIONS = 256
+
+
+def key_slices(n_tiles: int, longest: int, one_token_each: bool) -> int:
+    """Into how many slices the matrix-core kernel cuts each tile's keys (a workgroup each): enough for
+    WORKGROUPS_WANTED workgroups, no slice shorter than a few rounds, a power of two, 64 at most.  Measured at 16
+    heads of 128: a prompt of 2,048 tokens 322 / 186 / 130 / 152 us in 1 / 2 / 4 / 8 slices (the parts of more slices
+    cost the second kernel more than they even out), eight requests of one token on 2,048 keys 304 / 50 / 23 / 31 us
+    in 1 / 8 / 32 / 64."""
+    least = MIN_KEYS_PER_SLICE if one_token_each else MIN_KEYS_PER_SLICE_OF_PORTIONS
+    n = max(1, min(-(-WORKGROUPS_WANTED // max(1, n_tiles)), longest // least, 64))
+    return 1 << (n.bit_length() - 1)
 
 
 register_part("mixer", "talking_attention", TalkingAttention)
