@@ -223,9 +223,15 @@ extern "C" int ix_attention_talk_plain(const void* q, const void* k_cache, const
   IX_REQUIRE(window >= 0, "window must not be negative");
   const size_t lds = (static_cast<size_t>(heads) * head_dim + static_cast<size_t>(talk ? 2 : 1) * heads * TALK_CHUNK +
                       static_cast<size_t>(heads) * heads + 3 * heads + TALK_CHUNK) * sizeof(float);
-  IX_REQUIRE(lds <= 64 * 1024, "queries and scores of one token do not fit 64 KB of LDS");
+  IX_REQUIRE(lds <= 128 * 1024, "queries and scores of one token do not fit 128 KB of LDS");
   if (tokens == 0) return 0;
   dim3 grid(tokens), block(TALK_THREADS);
+  if (lds > 64 * 1024) {  // more than 64 KB of LDS for a workgroup has to be allowed per kernel
+    const void* fn = dtype == IX_F32 ? reinterpret_cast<const void*>(&attn_talk_plain_kernel<float>)
+                                     : reinterpret_cast<const void*>(&attn_talk_plain_kernel<bf16_t>);
+    IX_REQUIRE(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) == hipSuccess,
+               "the kernel was refused more than 64 KB of LDS");
+  }
   if (dtype == IX_F32)
     hipLaunchKernelGGL(attn_talk_plain_kernel<float>, grid, block, lds, stream, (const float*)q, (const float*)k_cache,
                        (const float*)v_cache, block_table, seq_of_token, positions, (float*)out, talk, sink,

@@ -16,7 +16,7 @@ import tiny_pelalix as tp
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LENGTHS = {"P": (5, 9, 17, 70), "Q": (7, 23, 40, 75), "R": (3, 50, 66), "S": (1, 2, 33, 70)}
+LENGTHS = {"P": (5, 9, 17, 70), "Q": (7, 23, 40, 75), "R": (3, 50, 66), "S": (1, 2, 33, 70), "U": (4, 19, 45)}
 # relative to the largest |logit| of the expected rows; fixed before the first run
 TOL = {"float32": ru.FP32_TOL, "bfloat16": ru.BF16_TOL}
 
@@ -60,7 +60,7 @@ WAYS = {"whole": lambda p: ru.whole(p), "tail": lambda p: ru.tail_decoded(p, 32)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "U"])
 @pytest.mark.parametrize("way", ["whole", "tail", "portions"])
 def test_each_request_alone(folders, name, dtype, way):
     runner = make_runner(folders, name, dtype)
@@ -70,7 +70,7 @@ def test_each_request_alone(folders, name, dtype, way):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "U"])
 def test_mixed_batches_with_few_pages(folders, name, dtype):
     """Up to four live requests, portions of some beside single tokens of others, in a pool with room for about two
     of the longer ones: pages and state slots are given back and used again, and that must happen for the run to

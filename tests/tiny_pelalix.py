@@ -27,7 +27,10 @@ Q = _config(131, 72, 1.0, 1e-6, [_layer(4, 1, 24, 40, 0.3, False, 100), _layer(4
 R = _config(256, 128, 8.0, 1e-5, [_layer(2, 2, 64, 64, 0.125, True, 256)])
 # S: a single head
 S = _config(97, 40, 2.0, 1e-5, [_layer(1, 1, 16, 16, 0.25, True, 64), _layer(1, 1, 16, 16, 0.25, True, 64)])
-CONFIGS = {"P": P, "Q": Q, "R": R, "S": S}
+# U: nothing is a multiple of 4 where the design allows it; the embedding's scale is left to its default
+U = _config(77, 90, 1.0, 1e-5, [_layer(3, 1, 20, 12, 0.22, True, 50), _layer(6, 1, 20, 12, 0.3, True, 70)])
+del U["embedding"]
+CONFIGS = {"P": P, "Q": Q, "R": R, "S": S, "U": U}
 
 
 def make_folder(raw_config: dict, seed: int, out_dir: str, dtype: str = "bfloat16") -> str:
