@@ -556,7 +556,7 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--prefill-tokens", type=int, default=PROMPT,
-                    help="tokens of the prompt whose reading in one step is timed (2,048 is the contract's)")
+                    help="tokens of the prompt whose reading in one step is timed (2,048 is the default workload's)")
     ap.add_argument("--prefill-context", type=int, default=0,
                     help="portion: tokens that the request has read before the timed portion")
     ap.add_argument("--shape", default="a27b", choices=["a27b", "57b"], help="portion: whose layer sizes")
