@@ -45,7 +45,7 @@ def host_lib():
         i32p, i64p = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64)
         vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
         sig = {
-            "ixh_cache_create": (vp, [ci, i32p, i32p, ci, ci, i64, i64]),
+            "ixh_cache_create": (vp, [ci, i32p, i32p, i32p, ci, ci, i64, i64]),
             "ixh_cache_destroy": (None, [vp]),
             "ixh_cache_error": (ctypes.c_char_p, [vp]),
             "ixh_cache_max_blocks": (ci, [vp]),
@@ -141,10 +141,12 @@ class GroupLayout:
     """One page group: `window` 0 keeps every token, W > 0 only the last W.  `release_passed` False keeps the
     pages that the window has passed until the request ends (what the reference does for its windowed layers,
     src/model/gpt_oss.cc:259-262); the attention kernels mask by the window either way, so the two settings must
-    give the same logits, which is what the switch is for."""
+    give the same logits, which is what the switch is for.  `keep_first`: the pages that hold a request's first
+    `keep_first` tokens are never given back (a window whose queries also read those tokens)."""
 
     window: int = 0
     release_passed: bool = True
+    keep_first: int = 0
 
     @property
     def release_window(self) -> int:
@@ -181,11 +183,13 @@ RESERVE_OK, RESERVE_POOL_EMPTY, RESERVE_CONTEXT_FULL = "ok", "pool_empty", "cont
 _RESERVE = {0: RESERVE_OK, 1: RESERVE_POOL_EMPTY, 2: RESERVE_CONTEXT_FULL}
 
 
-def pages_for_window(window: int, page_size: int, max_requests: int, max_step_tokens: int) -> int:
+def pages_for_window(window: int, page_size: int, max_requests: int, max_step_tokens: int,
+                     keep_first: int = 0) -> int:
     """Pages that a windowed group can ever hold at once when no step brings more than `max_step_tokens` tokens
     of a request: per request the pages that cover the window behind its next position and the step in front of
-    it (plus the two that the ends may straddle), for every request slot.  A pool of this size never runs out."""
-    return max_requests * (-(-(window + max_step_tokens) // page_size) + 2)
+    it (plus the two that the ends may straddle) and the pages of the `keep_first` tokens that are never given
+    back, for every request slot.  A pool of this size never runs out."""
+    return max_requests * (-(-(window + max_step_tokens) // page_size) + 2 + -(-keep_first // page_size))
 
 
 class CacheManager:
@@ -212,9 +216,10 @@ class CacheManager:
         self._lib = host_lib()
         G = len(self.groups)
         windows = (ctypes.c_int32 * max(G, 1))(*[g.release_window for g in self.groups])
+        keeps = (ctypes.c_int32 * max(G, 1))(*[g.keep_first for g in self.groups])
         pages = (ctypes.c_int32 * max(G, 1))(*pages_per_group)
         self.max_step_tokens = max_step_tokens
-        self._h = self._lib.ixh_cache_create(G, windows, pages, page_size, max_requests, max_seq_len,
+        self._h = self._lib.ixh_cache_create(G, windows, keeps, pages, page_size, max_requests, max_seq_len,
                                              int(max_step_tokens or 0))
         if not self._h:
             raise CacheError("the cache manager could not be created")

@@ -6,9 +6,11 @@ from . import qwen2_moe  # registers Qwen2MoeForCausalLM
 from .qwen2_moe import Qwen2MoeConfig
 from . import pelalix  # registers Pelalix
 from .pelalix import PelalixConfig
+from . import dezudra  # registers Dezudra
+from .dezudra import DezudraConfig
 
 __all__ = [
     "ConfigError", "config_class_for", "config_from_dict", "config_from_directory", "config_from_json",
     "known_architectures", "register_architecture", "LayerSpec", "ModelSpec", "PartSpec", "ScheduleEntry", "linear_head", "token_embedding",
-    "Qwen2MoeConfig", "PelalixConfig",
+    "Qwen2MoeConfig", "PelalixConfig", "DezudraConfig",
 ]

@@ -99,7 +99,10 @@ def token_embedding(name: str, vocab_size: int, hidden_size: int, init_std: floa
                                         "init_std": init_std}, rename={"weight": name})
 
 
-def linear_head(name: str, vocab_size: int, hidden_size: int, init_std: float = 0.02) -> PartSpec:
-    """The usual head: logits = x . W^T with W = `name` of [vocab, hidden]; a tied head names the embedding's table."""
-    return PartSpec("linear_head", {"vocab_size": vocab_size, "hidden_size": hidden_size, "init_std": init_std},
-                    rename={"weight": name})
+def linear_head(name: str, vocab_size: int, hidden_size: int, init_std: float = 0.02, scale: float = 1.0) -> PartSpec:
+    """The usual head: logits = x . W^T * scale with W = `name` of [vocab, hidden]; a tied head names the embedding's
+    table."""
+    params = {"vocab_size": vocab_size, "hidden_size": hidden_size, "init_std": init_std}
+    if scale != 1.0:
+        params["scale"] = scale
+    return PartSpec("linear_head", params, rename={"weight": name})

@@ -50,6 +50,7 @@ struct Request {
 
 struct Cache {
   std::vector<int32_t> windows;
+  std::vector<int32_t> keeps;  // per group: the first tokens of a request that a windowed group never gives back
   std::vector<Pool> pools;
   int32_t page_size = 0, max_requests = 0, max_blocks = 0;
   int64_t max_seq_len = 0;
@@ -95,7 +96,8 @@ struct Cache {
       auto& b = r.blocks[g];
       int64_t first = first_live_page(g, r.cached);
       if (first > static_cast<int64_t>(b.size())) first = static_cast<int64_t>(b.size());
-      for (int64_t j = 0; j < first; ++j)
+      // pages that hold one of the kept first tokens stay as long as the request lives
+      for (int64_t j = (keeps[g] + page_size - 1) / page_size; j < first; ++j)
         if (b[static_cast<size_t>(j)] >= 0) {
           ok = release_page(g, b[static_cast<size_t>(j)]) && ok;
           b[static_cast<size_t>(j)] = -1;
@@ -138,13 +140,14 @@ Cache* C(void* h) { return static_cast<Cache*>(h); }
 
 extern "C" {
 
-void* ixh_cache_create(int n_groups, const int32_t* windows, const int32_t* pages, int page_size, int max_requests,
-                       int64_t max_seq_len, int64_t step_cap) {
+void* ixh_cache_create(int n_groups, const int32_t* windows, const int32_t* keeps, const int32_t* pages, int page_size,
+                       int max_requests, int64_t max_seq_len, int64_t step_cap) {
   if (n_groups < 0 || page_size <= 0 || max_requests <= 0 || max_seq_len <= 0 || step_cap < 0) return nullptr;
   for (int g = 0; g < n_groups; ++g)
-    if (pages[g] <= 0) return nullptr;
+    if (pages[g] <= 0 || keeps[g] < 0) return nullptr;
   Cache* c = new Cache();
   c->windows.assign(windows, windows + n_groups);
+  c->keeps.assign(keeps, keeps + n_groups);
   for (int g = 0; g < n_groups; ++g) c->pools.emplace_back(pages[g]);
   c->page_size = page_size;
   c->max_requests = max_requests;

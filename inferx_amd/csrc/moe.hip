@@ -26,7 +26,8 @@
 // them like the chosen ones.
 __device__ __forceinline__ void route_select(float* z, float* red, float* __restrict__ topk_w,
                                              int32_t* __restrict__ topk_e, int64_t t, int experts, int k,
-                                             int renormalize, float scale, int always = 0, float always_w = 1.0f) {
+                                             int renormalize, float scale, int always = 0, float always_w = 1.0f,
+                                             int n_groups = 1, int groups_keep = 1) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   float mx = -INFINITY;
   for (int e = tid; e < experts; e += blockDim.x) mx = fmaxf(mx, z[e]);
@@ -40,6 +41,29 @@ __device__ __forceinline__ void route_select(float* z, float* red, float* __rest
   sum = ix_block_sum(sum, red);  // its barriers also publish z
   if (wave != 0) return;
   const float inv_sum = 1.0f / sum;
+  if (groups_keep < n_groups) {
+    // The experts form n_groups equal groups of neighbours (at most 64), a group's score is its largest score, and
+    // only experts of the groups_keep best groups can be chosen (among equal groups the lower number first): the
+    // others' scores are struck out before the rounds below.  The weights stay the scores over all experts.
+    const int per = experts / n_groups;
+    float best = -INFINITY;
+    if (lane < n_groups)
+      for (int e = lane * per; e < (lane + 1) * per; ++e) best = fmaxf(best, z[e]);
+    bool kept = false;
+    for (int round = 0; round < groups_keep; ++round) {
+      float bv = best;
+      int bi = lane < n_groups ? lane : 0x7fffffff;
+      ix_wave_argmax(bv, bi);
+      if (lane == bi) {
+        kept = true;
+        best = -INFINITY;
+      }
+    }
+    if (lane < n_groups && !kept)
+      for (int e = lane * per; e < (lane + 1) * per; ++e) z[e] = -INFINITY;
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+  }
   float chosen = 0.f;  // lane s keeps the weight of slot s
   float total = 0.f;
   for (int slot = 0; slot < k; ++slot) {
@@ -75,7 +99,7 @@ __global__ void __launch_bounds__(ROUTE_THREADS)
 moe_route_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dtype,
                  const void* __restrict__ shared_gate_w, int sg_dtype, float* __restrict__ topk_w,
                  int32_t* __restrict__ topk_e, float* __restrict__ shared_gate, int64_t width, int experts, int k,
-                 int renormalize, float scale, int always) {
+                 int renormalize, float scale, int always, int n_groups, int groups_keep) {
   extern __shared__ __align__(16) float smem[];
   float* xs = smem;                        // [width rounded up to 4]
   float* z = smem + ((width + 3) & ~3);    // [experts + 1]
@@ -94,7 +118,7 @@ moe_route_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dt
   __syncthreads();
   const float gate = shared_gate_w ? 1.0f / (1.0f + expf(-z[experts])) : 1.0f;
   if (shared_gate_w && tid == 0) shared_gate[t] = gate;
-  route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale, always, gate);
+  route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale, always, gate, n_groups, groups_keep);
 }
 
 // Few tokens (decoding): the router rows are spread over many workgroups, one row per wavefront,
@@ -121,7 +145,7 @@ moe_route_logits_kernel(const T* __restrict__ x, const void* __restrict__ wr, in
 __global__ void __launch_bounds__(64)
 moe_route_select_kernel(const float* __restrict__ logits, float* __restrict__ topk_w, int32_t* __restrict__ topk_e,
                         float* __restrict__ shared_gate, int experts, int k, int renormalize, float scale,
-                        int always) {
+                        int always, int n_groups, int groups_keep) {
   extern __shared__ __align__(16) float z[];  // [experts]
   __shared__ float red[16];
   const int64_t t = blockIdx.x;
@@ -129,7 +153,7 @@ moe_route_select_kernel(const float* __restrict__ logits, float* __restrict__ to
   const float gate = shared_gate ? 1.0f / (1.0f + expf(-logits[t * (experts + 1) + experts])) : 1.0f;
   if (shared_gate && threadIdx.x == 0) shared_gate[t] = gate;
   __syncthreads();
-  route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale, always, gate);
+  route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale, always, gate, n_groups, groups_keep);
 }
 
 // Many tokens, bfloat16 activations and weights: the scores on the matrix cores (exact products of bfloat16
@@ -185,8 +209,11 @@ moe_route_logits_mfma_kernel(const __bf16* __restrict__ x, const __bf16* __restr
 extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dtype, const void* shared_gate_w,
                             int sg_dtype, float* topk_w, int32_t* topk_e, float* shared_gate, float* logits_scratch,
                             int64_t tokens, int64_t width, int experts, int k, int renormalize, float scale,
-                            int always, hipStream_t stream) {
+                            int always, int n_groups, int groups_keep, hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
+  IX_REQUIRE(n_groups >= 1 && n_groups <= 64 && experts % n_groups == 0 && groups_keep >= 1 && groups_keep <= n_groups,
+             "between 1 and 64 equal groups of experts, of which between 1 and all are kept");
+  IX_REQUIRE(k <= static_cast<int64_t>(groups_keep) * (experts / n_groups), "top_k must fit into the kept groups");
   IX_REQUIRE(always >= 0 && always <= 32 && experts + always <= IX_MAX_EXPERTS,
              "between 0 and 32 experts that every token uses, within the limit of all experts");
   IX_REQUIRE(experts > 0 && experts <= IX_MAX_EXPERTS, "number of experts must be between 1 and 1024");
@@ -207,7 +234,7 @@ extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dty
                          wr_dtype, shared_gate_w, sg_dtype, logits_scratch, width, experts);
     hipLaunchKernelGGL(moe_route_select_kernel, dim3(tokens), dim3(64), experts * sizeof(float), stream,
                        logits_scratch, topk_w, topk_e, shared_gate_w ? shared_gate : nullptr, experts, k, renormalize,
-                       scale, always);
+                       scale, always, n_groups, groups_keep);
     return ix_check_launch("ix_moe_route");
   }
   if (logits_scratch != nullptr && dtype == IX_BF16 && wr_dtype == IX_BF16 &&
@@ -219,18 +246,18 @@ extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dty
                        tokens, (int)width, experts);
     hipLaunchKernelGGL(moe_route_select_kernel, dim3(tokens), dim3(64), experts * sizeof(float), stream,
                        logits_scratch, topk_w, topk_e, shared_gate_w ? shared_gate : nullptr, experts, k, renormalize,
-                       scale, always);
+                       scale, always, n_groups, groups_keep);
     return ix_check_launch("ix_moe_route");
   }
   dim3 grid(tokens), block(ROUTE_THREADS);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, smem, stream, (const float*)x, wr, wr_dtype,
                        shared_gate_w, sg_dtype, topk_w, topk_e, shared_gate, width, experts, k, renormalize, scale,
-                       always);
+                       always, n_groups, groups_keep);
   else
     hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, block, smem, stream, (const bf16_t*)x, wr, wr_dtype,
                        shared_gate_w, sg_dtype, topk_w, topk_e, shared_gate, width, experts, k, renormalize, scale,
-                       always);
+                       always, n_groups, groups_keep);
   return ix_check_launch("ix_moe_route");
 }
 
@@ -373,7 +400,7 @@ template <typename TA, typename TW, typename TO, bool GATE_UP>
 __global__ void __launch_bounds__(256)
 moe_grouped_plain_kernel(const TA* __restrict__ a, const TW* __restrict__ w, TO* __restrict__ out,
                          const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows, int experts,
-                         int64_t n_out, int64_t width) {
+                         int64_t n_out, int64_t width, int act) {
   __shared__ float As[GG_BK][GG_BM + 4];
   __shared__ float Ws[GATE_UP ? 2 : 1][GG_BK][GG_BN + 4];
   __shared__ int32_t src_row[GG_BM];
@@ -450,6 +477,7 @@ moe_grouped_plain_kernel(const TA* __restrict__ a, const TW* __restrict__ w, TO*
       if (n >= n_out) continue;
       float v = acc[0][i][j];
       if (GATE_UP) v = v / (1.0f + expf(-v)) * acc[1][i][j];
+      else if (act) v = v > 0.f ? v * v : 0.f;  // the square of relu
       ix_store(out + static_cast<int64_t>(r) * n_out + n, v);
     }
   }
@@ -458,12 +486,12 @@ moe_grouped_plain_kernel(const TA* __restrict__ a, const TW* __restrict__ w, TO*
 template <bool GATE_UP>
 static int launch_grouped_plain(const void* a, int a_dtype, const void* w, int w_dtype, void* out,
                                 const int32_t* offsets, const int32_t* rows, int64_t assignments, int experts,
-                                int64_t n_out, int64_t width, hipStream_t stream) {
+                                int64_t n_out, int64_t width, int act, hipStream_t stream) {
   const int64_t m_tiles = std::min<int64_t>(assignments, (assignments + GG_BM - 1) / GG_BM + experts);
   dim3 grid((n_out + GG_BN - 1) / GG_BN, m_tiles), block(256);
 #define LAUNCH(TA, TW)                                                                                            \
   hipLaunchKernelGGL((moe_grouped_plain_kernel<TA, TW, TA, GATE_UP>), grid, block, 0, stream, (const TA*)a,        \
-                     (const TW*)w, (TA*)out, offsets, rows, experts, n_out, width)
+                     (const TW*)w, (TA*)out, offsets, rows, experts, n_out, width, act)
   if (a_dtype == IX_F32 && w_dtype == IX_F32) LAUNCH(float, float);
   else if (a_dtype == IX_F32 && w_dtype == IX_BF16) LAUNCH(float, bf16_t);
   else if (a_dtype == IX_BF16 && w_dtype == IX_F32) LAUNCH(bf16_t, float);
@@ -479,10 +507,11 @@ extern "C" int ix_moe_grouped_plain(const void* a, int a_dtype, const void* w, i
   IX_REQUIRE(assignments >= 0 && n_out > 0 && width > 0 && experts > 0, "sizes must be positive");
   IX_REQUIRE(assignments < (1ll << 31) / GG_BM, "too many assignments");
   if (assignments == 0) return 0;
-  return gate_up ? launch_grouped_plain<true>(a, a_dtype, w, w_dtype, out, offsets, rows, assignments, experts, n_out,
-                                              width, stream)
-                 : launch_grouped_plain<false>(a, a_dtype, w, w_dtype, out, offsets, rows, assignments, experts,
-                                               n_out, width, stream);
+  IX_REQUIRE(gate_up >= 0 && gate_up <= 2, "gate_up must be 0 (plain), 1 (gate|up with SwiGLU) or 2 (square of relu)");
+  return gate_up == 1 ? launch_grouped_plain<true>(a, a_dtype, w, w_dtype, out, offsets, rows, assignments, experts,
+                                                   n_out, width, 0, stream)
+                      : launch_grouped_plain<false>(a, a_dtype, w, w_dtype, out, offsets, rows, assignments, experts,
+                                                    n_out, width, gate_up == 2 ? 1 : 0, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -31,7 +31,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 template <int MT, bool GATE_UP, int KSPLIT, typename TO = __bf16, int NB = 1>
 __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
                                              TO* __restrict__ out, const int32_t* __restrict__ rows, int e,
-                                             int row0, int row_end, int n0, int n_out, int width, float* red) {
+                                             int row0, int row_end, int n0, int n_out, int width, float* red,
+                                             int act = 0) {
   constexpr int NACC = NB * (GATE_UP ? 2 : 1);  // accumulator b + NB h: block b of the gate (h = 0) or up (1) rows
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int m = lane & 15, g = lane >> 4;
@@ -156,6 +157,7 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
       for (int i = 0; i < 4; ++i) {
         v[i] = acc[u][t][i];
         if constexpr (GATE_UP) v[i] = v[i] / (1.0f + __expf(-v[i])) * acc[NB + u][t][i];
+        else if (act) v[i] = v[i] > 0.f ? v[i] * v[i] : 0.f;  // the square of relu
       }
       TO* dst = out + static_cast<int64_t>(r) * n_out + nb;
       if (nb + 4 <= n_out && (n_out & 3) == 0) {
@@ -190,13 +192,14 @@ __global__ void __launch_bounds__(256)
 moe_grouped_mfma_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ out,
                         const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
                         const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
-                        const int32_t* __restrict__ tile_info, int n_out, int width) {
+                        const int32_t* __restrict__ tile_info, int n_out, int width, int act) {
   __shared__ float red[KSPLIT > 1 ? 3 * 64 * MT * (GATE_UP ? 2 : 1) * 4 : 1];
   if (static_cast<int>(blockIdx.y) >= tile_info[0]) return;
   const int e = tile_expert[blockIdx.y];
   const int n0 = (KSPLIT > 1 ? blockIdx.x : blockIdx.x * 4 + (threadIdx.x >> 6)) * 16;
   if (n0 >= n_out) return;  // whole wavefront (KSPLIT == 1) or whole workgroup
-  grouped_body<MT, GATE_UP, KSPLIT>(a, w, out, rows, e, tile_row0[blockIdx.y], offsets[e + 1], n0, n_out, width, red);
+  grouped_body<MT, GATE_UP, KSPLIT>(a, w, out, rows, e, tile_row0[blockIdx.y], offsets[e + 1], n0, n_out, width, red,
+                                    act);
 }
 
 // Routed experts and the shared expert in one launch (decoding: every launch saved counts).  The first
@@ -232,7 +235,8 @@ moe_grouped_dual_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ o
 }
 
 // `max_tiles` bounds the number of row tiles (the grid); the kernel reads the true number from tile_info.
-// tile_rows (16, 32 or 64) must be what the grouping kernel was given.
+// tile_rows (16, 32 or 64) must be what the grouping kernel was given.  gate_up: 0 a plain product, 1 gate|up rows
+// with SwiGLU, 2 a plain product whose results pass the square of relu.
 extern "C" int ix_moe_grouped_mfma(const void* a, const void* w, void* out, const int32_t* offsets,
                                    const int32_t* rows, const int32_t* tile_expert, const int32_t* tile_row0,
                                    const int32_t* tile_info, int max_tiles, int tile_rows, int64_t n_out,
@@ -242,6 +246,7 @@ extern "C" int ix_moe_grouped_mfma(const void* a, const void* w, void* out, cons
   IX_REQUIRE(n_out < (1 << 30) && width < (1 << 30), "sizes too large");
   IX_REQUIRE(tile_rows == 16 || tile_rows == 32 || tile_rows == 64, "tile_rows must be 16, 32 or 64");
   IX_REQUIRE(k_split == 1 || k_split == 4, "k_split must be 1 or 4");
+  IX_REQUIRE(gate_up >= 0 && gate_up <= 2, "gate_up must be 0, 1 or 2");
   IX_REQUIRE(max_tiles <= 65535, "too many row tiles for one launch");
   if (max_tiles == 0) return 0;
   const int n_tiles16 = static_cast<int>((n_out + 15) / 16);
@@ -249,9 +254,9 @@ extern "C" int ix_moe_grouped_mfma(const void* a, const void* w, void* out, cons
 #define LAUNCH(MT, GU, KS)                                                                                        \
   hipLaunchKernelGGL((moe_grouped_mfma_kernel<MT, GU, KS>), grid, block, 0, stream, (const __bf16*)a,             \
                      (const __bf16*)w, (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, \
-                     (int)width)
+                     (int)width, gate_up == 2 ? 1 : 0)
 #define PICK(MT)                                       \
-  if (gate_up) {                                       \
+  if (gate_up == 1) {                                  \
     if (k_split > 1) LAUNCH(MT, true, 4);              \
     else LAUNCH(MT, true, 1);                          \
   } else {                                             \
@@ -290,7 +295,7 @@ extern "C" int ix_moe_grouped_dual(const void* a, const void* w, void* out, cons
                      (int)width, (const __bf16*)a_s, (const __bf16*)w_s, (__bf16*)out_s, shared_rows, (int)n_out_s, \
                      (int)width_s)
 #define PICK(MT, NB)                 \
-  if (gate_up) LAUNCH(MT, true, NB); \
+  if (gate_up == 1) LAUNCH(MT, true, NB); \
   else LAUNCH(MT, false, NB);
   if (tile_rows == 16) { PICK(1, 1) } else if (tile_rows == 32) { PICK(2, 1) } else { PICK(4, 1) }
 #undef PICK

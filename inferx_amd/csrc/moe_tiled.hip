@@ -54,7 +54,7 @@ __device__ __forceinline__ int tl_at(int row, int piece) { return row * TL_STRID
 template <bool GATE_UP, int NP, int NWW>
 __device__ __forceinline__ void
 tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ rows, int n_out, int width,
-           int e, int row0, int row_end, int tile, int col_block, __bf16* ws, __bf16* xs) {
+           int e, int row0, int row_end, int tile, int col_block, __bf16* ws, __bf16* xs, int act) {
   // (a and w are plain pointers on purpose: loads through `const __restrict__` ones may be moved by the
   // optimiser, which sinks them to their first use and so undoes the prefetch)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -265,14 +265,20 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int nb = n0 + 64 * wi + 16 * j + 4 * g;
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[i] = acc[j][t][i];
+          if (act) v[i] = v[i] > 0.f ? v[i] * v[i] : 0.f;  // the square of relu
+        }
         __bf16* dst = out + static_cast<int64_t>(r) * n_out + nb;
         if (nb + 4 <= n_out && vec) {
-          bf16x4 o = {(__bf16)acc[j][t][0], (__bf16)acc[j][t][1], (__bf16)acc[j][t][2], (__bf16)acc[j][t][3]};
+          bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
           *reinterpret_cast<bf16x4*>(dst) = o;
         } else {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
-            if (nb + i < n_out) dst[i] = (__bf16)acc[j][t][i];
+            if (nb + i < n_out) dst[i] = (__bf16)v[i];
         }
       }
     }
@@ -284,7 +290,8 @@ __global__ void __launch_bounds__(TL_THREADS(NWW)) __attribute__((amdgpu_waves_p
 moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ offsets,
                          const int32_t* __restrict__ rows,
                          const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
-                         const int32_t* __restrict__ tile_info, int n_out, int width, int n_col_blocks) {
+                         const int32_t* __restrict__ tile_info, int n_out, int width, int n_col_blocks,
+                         int act) {
   __shared__ __attribute__((aligned(16))) __bf16 ws[2 * TL_WTILE(NWW)];
   __shared__ __attribute__((aligned(16))) __bf16 xs[2 * TL_XTILE(NWW)];
   // Workgroups go to the chip's eight dies in turn, by their number.  All column blocks of a row tile read the
@@ -298,18 +305,19 @@ moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const in
   const int held = min(TL_ROWS(NWW), row_end - row0);
   if (held <= 0) return;
   switch ((held + 31) >> 5) {  // pairs of sixteens of rows this tile holds
-    case 1: tiled_body<GATE_UP, 1, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
-    case 2: tiled_body<GATE_UP, 2, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
-    case 3: tiled_body<GATE_UP, 3, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
-    case 4: tiled_body<GATE_UP, 4, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
-    case 5: tiled_body<GATE_UP, 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    case 1: tiled_body<GATE_UP, 1, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act); break;
+    case 2: tiled_body<GATE_UP, 2, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act); break;
+    case 3: tiled_body<GATE_UP, 3, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act); break;
+    case 4: tiled_body<GATE_UP, 4, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act); break;
+    case 5: tiled_body<GATE_UP, 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act); break;
     default:  // (six pairs of sixteens in the wide form only)
-      tiled_body<GATE_UP, NWW == 4 ? 6 : 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs);
+      tiled_body<GATE_UP, NWW == 4 ? 6 : 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs, act);
       break;
   }
 }
 
 // The row-tile map must have been made for tiles of 160 rows, for the wide form of 192.  `wide`: see below.
+// gate_up: 0 a plain product, 1 gate|up rows with SwiGLU, 2 a plain product whose results pass the square of relu.
 extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, const int32_t* offsets,
                                     const int32_t* rows, const int32_t* tile_expert, const int32_t* tile_row0,
                                     const int32_t* tile_info, int max_tiles, int64_t a_rows, int64_t n_out,
@@ -317,7 +325,7 @@ extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, con
   IX_REQUIRE(n_out > 0 && width > 0 && max_tiles >= 0, "sizes must be positive");
   IX_REQUIRE(width % 8 == 0, "the reduction width must be a multiple of 8 for the matrix-core kernel");
   IX_REQUIRE(n_out < (1 << 30) && width < (1 << 30), "sizes too large");
-  IX_REQUIRE(a_rows >= 0 && a_rows * width < (int64_t(1) << 31) && (gate_up ? 2 : 1) * n_out * width < (int64_t(1) << 31),
+  IX_REQUIRE(a_rows >= 0 && a_rows * width < (int64_t(1) << 31) && (gate_up == 1 ? 2 : 1) * n_out * width < (int64_t(1) << 31),
              "the activations, and one expert's weights, must hold fewer than 2^31 numbers");
   IX_REQUIRE(max_tiles <= 65535, "too many row tiles for one launch");
   if (max_tiles == 0) return 0;
@@ -325,7 +333,7 @@ extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, con
   // workgroup per compute unit): the activations are staged for half as many column blocks.  Same sums in the
   // same order either way.
   const int nww = wide ? 4 : 2;
-  const int cols = gate_up ? 32 * nww : 64 * nww;
+  const int cols = gate_up == 1 ? 32 * nww : 64 * nww;
   const int n_col_blocks = static_cast<int>((n_out + cols - 1) / cols);
   const int64_t groups = 8 * static_cast<int64_t>(n_col_blocks) * ((max_tiles + 7) / 8);
   IX_REQUIRE(groups < (int64_t(1) << 31), "too many workgroups for one launch");
@@ -333,12 +341,12 @@ extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, con
 #define LAUNCH(GU, NWW)                                                                                             \
   hipLaunchKernelGGL((moe_grouped_tiled_kernel<GU, NWW>), grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w, \
                      (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, (int)width,         \
-                     n_col_blocks)
+                     n_col_blocks, gate_up == 2 ? 1 : 0)
   if (nww == 4) {
-    if (gate_up) LAUNCH(true, 4);
+    if (gate_up == 1) LAUNCH(true, 4);
     else LAUNCH(false, 4);
   } else {
-    if (gate_up) LAUNCH(true, 2);
+    if (gate_up == 1) LAUNCH(true, 2);
     else LAUNCH(false, 2);
   }
 #undef LAUNCH

@@ -128,7 +128,7 @@ class ModelRunner:
                 bound[name] = b
             self.bindings.append(bound)
         self._states = [b.state for bound in self.bindings for b in bound.values() if b.state is not None]
-        self.cache = CacheManager([GroupLayout(n.window, self.release_window_pages) for n in needs],
+        self.cache = CacheManager([GroupLayout(n.window, self.release_window_pages, n.keep_first) for n in needs],
                                   self.group_pages, self.page_size, self.max_requests, self.max_seq_len,
                                   self.max_step_tokens)
         self._graphs: Dict[Tuple[int, int], "_DecodeGraph"] = {}
@@ -143,7 +143,8 @@ class ModelRunner:
         """A group that keeps every token gets `num_pages`; a windowed one that gives passed pages back, when the
         largest step is known, no more than it can ever hold."""
         if need.window > 0 and self.release_window_pages and self.max_step_tokens:
-            return min(num_pages, pages_for_window(need.window, self.page_size, self.max_requests, self.max_step_tokens))
+            return min(num_pages, pages_for_window(need.window, self.page_size, self.max_requests, self.max_step_tokens,
+                                                    need.keep_first))
         return num_pages
 
     def kv_bytes_per_token(self) -> int:

@@ -316,15 +316,19 @@ ROUTE_SMALL_TOKENS = 128
 
 def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor], topk_w: torch.Tensor,
               topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor], renormalize: bool, scale: float,
-              always: int = 0) -> None:
+              always: int = 0, groups: int = 1, groups_keep: int = 1) -> None:
     """Router product, softmax and top-k in float32; optional sigmoid gate of the shared expert.
     `always`: that many further slots per token after the chosen ones (topk_w and topk_e are [T, k + always]), naming
-    the experts E .. E + always - 1 with the shared gate's value (or 1) as their weight: experts that every token uses."""
+    the experts E .. E + always - 1 with the shared gate's value (or 1) as their weight: experts that every token uses.
+    `groups`, `groups_keep`: the experts form that many equal groups of neighbours, and only experts of the
+    `groups_keep` groups with the largest best score can be chosen (1, 1: every expert can)."""
     T, H = x.shape
     E = router_w.shape[0]
     k = topk_w.shape[1] - always
     _need(router_w.shape == (E, H), "router weight must be [experts, hidden]")
     _need(k > 0 and always >= 0, "at least one chosen slot")
+    _need(1 <= groups <= 64 and E % groups == 0 and 1 <= groups_keep <= groups and k <= groups_keep * (E // groups),
+          "the experts must split into at most 64 equal groups, and the kept groups must hold top_k experts")
     _need(topk_w.shape == (T, k + always) and topk_w.dtype == torch.float32, "topk_w must be float32 [T, k + always]")
     _need(topk_e.shape == (T, k + always) and topk_e.dtype == torch.int32, "topk_e must be int32 [T, k + always]")
     if shared_gate_w is not None:
@@ -341,7 +345,7 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[t
     _call("ix_moe_route", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)), _ptr(shared_gate_w),
           _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(topk_w), _ptr(topk_e),
           _ptr(shared_gate if shared_gate_w is not None else None), _ptr(scratch), _i64(T), _i64(H), _i32(E), _i32(k),
-          _i32(1 if renormalize else 0), _f32(scale), _i32(always), _stream())
+          _i32(1 if renormalize else 0), _f32(scale), _i32(always), _i32(groups), _i32(groups_keep), _stream())
 
 
 # the one-launch router: at most this many tokens, experts and bytes of one token as float32
@@ -441,6 +445,17 @@ def moe_dispatch(topk_e: torch.Tensor, offsets: torch.Tensor, rows: torch.Tensor
           _i32(tile_rows), _ptr(te), _ptr(tr), _ptr(ti), _stream())
 
 
+PLAIN_PRODUCT, GATE_UP_SWIGLU, RELU_SQUARED = 0, 1, 2
+
+
+def _epilogue(gate_up) -> int:
+    """What a grouped product does with its sums: False / 0 nothing, True / 1 the weights hold gate rows then up rows
+    and the result is silu(gate) * up, 2 the square of relu of a plain product."""
+    code = int(gate_up)
+    _need(code in (PLAIN_PRODUCT, GATE_UP_SWIGLU, RELU_SQUARED), "unknown epilogue of a grouped product")
+    return code
+
+
 def moe_max_tiles(assignments: int, experts: int, tile_rows: int) -> int:
     """Upper bound of the number of row tiles: every expert may end with a partial tile."""
     return max(1, min(assignments, -(-assignments // tile_rows) + experts))
@@ -455,7 +470,7 @@ def moe_grouped_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offset
     K = a.shape[1]
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
           "the matrix-core grouped product is bfloat16 only")
-    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if gate_up else n_out),
+    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if _epilogue(gate_up) == GATE_UP_SWIGLU else n_out),
           "expert weight shape does not fit")
     _need(K % 8 == 0, "the reduction width must be a multiple of 8")
     _is_i32(offsets, E + 1)
@@ -467,7 +482,7 @@ def moe_grouped_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offset
     _is_i32(tile_map, 2 * mt + 1)
     _call("ix_moe_grouped_mfma", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
           _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i32(tile_rows), _i64(n_out), _i64(K),
-          _i32(1 if gate_up else 0), _i32(k_split), _stream())
+          _i32(_epilogue(gate_up)), _i32(k_split), _stream())
 
 
 def moe_grouped_dual(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
@@ -482,7 +497,7 @@ def moe_grouped_dual(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offset
     K_s = a_s.shape[1]
     for t in (a, w, out, a_s, w_s, out_s):
         _need(t.dtype == torch.bfloat16, "the matrix-core grouped product is bfloat16 only")
-    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if gate_up else n_out),
+    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if _epilogue(gate_up) == GATE_UP_SWIGLU else n_out),
           "expert weight shape does not fit")
     _need(w_s.shape == ((2 * n_out_s if gate_up else n_out_s), K_s) and a_s.shape[0] == T,
           "shared weight shape does not fit")
@@ -553,7 +568,7 @@ def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offse
     K = a.shape[1]
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
           "the matrix-core grouped product is bfloat16 only")
-    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if gate_up else n_out),
+    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if _epilogue(gate_up) == GATE_UP_SWIGLU else n_out),
           "expert weight shape does not fit")
     _need(K % 8 == 0, "the reduction width must be a multiple of 8")
     _is_i32(offsets, E + 1)
@@ -565,7 +580,7 @@ def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offse
     _is_i32(tile_map, 2 * mt + 1)
     _call("ix_moe_grouped_tiled", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
           _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i64(a.shape[0]), _i64(n_out), _i64(K),
-          _i32(1 if gate_up else 0), _i32(1 if wide else 0), _stream())
+          _i32(_epilogue(gate_up)), _i32(1 if wide else 0), _stream())
 
 
 def moe_grouped_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
@@ -575,7 +590,7 @@ def moe_grouped_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offse
     E = w.shape[0]
     A, n_out = out.shape
     K = a.shape[1]
-    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if gate_up else n_out),
+    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if _epilogue(gate_up) == GATE_UP_SWIGLU else n_out),
           "expert weight shape does not fit")
     _need(out.dtype == a.dtype, "out must have the activations' dtype")
     _is_i32(offsets, E + 1)
@@ -584,7 +599,7 @@ def moe_grouped_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offse
     else:
         _need(a.shape[0] >= A, "a has fewer rows than out")
     _call("ix_moe_grouped_plain", _ptr(a), _i32(_dt(a)), _ptr(w), _i32(_dt(w)), _ptr(out), _ptr(offsets), _ptr(rows),
-          _i64(A), _i32(E), _i64(n_out), _i64(K), _i32(1 if gate_up else 0), _stream())
+          _i64(A), _i32(E), _i64(n_out), _i64(K), _i32(_epilogue(gate_up)), _stream())
 
 
 def moe_combine(y: torch.Tensor, dest: torch.Tensor, topk_w: torch.Tensor, shared: Optional[torch.Tensor],
@@ -897,3 +912,145 @@ def attention_talk_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
           None if sink is None else _f32_vec(sink, heads, "the sinks"), gate_ptr, _i64(gate_stride), _i64(T),
           _i32(tiles.shape[1]), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(vd), _i32(k_cache.shape[2]),
           _i32(block_table.shape[1]), _f32(scale), _i32(heads_per_wave), _stream())
+
+
+# ---- layers that norm a branch's result as well, short convolutions, the delta rule, differential attention ------
+def add_normed_rmsnorm(h: torch.Tensor, delta: torch.Tensor, delta_weight: torch.Tensor, delta_eps: float,
+                       weight: Optional[torch.Tensor], out: Optional[torch.Tensor], eps: float,
+                       rows: Optional[torch.Tensor] = None) -> None:
+    """h += rmsnorm(delta) * delta_weight; out = rmsnorm(h) * weight, one pass.  With `rows`, out[r] comes from row
+    rows[r] and h stays as it was.  `weight` and `out` None: only the sum."""
+    H = h.shape[1]
+    _need(h.dtype == torch.float32, "the residual stream is float32")
+    _need(delta.shape == h.shape and delta_weight.numel() == H, "the branch's result must have the shape of h")
+    _need((weight is None) == (out is None), "a following norm and its output come together")
+    if out is not None:
+        _need(weight.numel() == H and out.shape[1] == H, "width mismatch")
+    n_out = h.shape[0] if out is None else out.shape[0]
+    if rows is None:
+        _need(n_out == h.shape[0], "out must have a row per row of h")
+    else:
+        _is_i32(rows, n_out)
+    _call("ix_add_normed_rmsnorm", _ptr(h), _ptr(delta), _i32(_dt(delta)), _ptr(delta_weight), _i32(_dt(delta_weight)),
+          _f32(delta_eps), _ptr(weight), _i32(_dt(weight) if weight is not None else F32), _f32(eps), _ptr(out),
+          _i32(_dt(out) if out is not None else F32), _ptr(rows), _i64(n_out), _i64(H), _stream())
+
+
+class StepRows:
+    """Where the rows of a step belong: what a kernel that carries something from a request's last step needs."""
+
+    def __init__(self, seq_of_token, q_start, state_slots):
+        self.seq_of_token, self.q_start, self.state_slots = seq_of_token, q_start, state_slots
+
+    def check(self, tokens: int) -> None:
+        _is_i32(self.seq_of_token, tokens)
+        _is_i32(self.q_start, 2)
+        _is_i32(self.state_slots, self.q_start.numel() - 1)
+
+
+def short_conv(x: torch.Tensor, bias: Optional[torch.Tensor], weight: torch.Tensor, state: torch.Tensor,
+               rows: StepRows, sizes: Tuple[int, int, int, int, int], out_q: torch.Tensor,
+               out_k: torch.Tensor, out_v: torch.Tensor, slots: Optional[torch.Tensor] = None,
+               cos_sin: Optional[torch.Tensor] = None, silu: bool = False) -> None:
+    """A causal convolution of `taps` = weight.shape[1] taps over time on the first q + k + v channels of x
+    [T, >= channels] (a bias added first), continued from `state` (a float32 view [slots, >= (taps - 1) * channels]
+    of each request's last inputs, brought up to date), then silu and / or the rotation of the first
+    2 * cos_sin.shape[1] elements of every q and k head.  `sizes` = (q channels, k channels, v channels, head_dim,
+    value_dim).  With `slots` k and v go into the paged caches out_k [pages, k heads, page, head_dim] and out_v
+    [pages, v heads, value_dim, page]; else to rows [T, k channels], [T, v channels].  q goes to out_q [T, q channels]."""
+    cq, ck, cv, d, vd = sizes
+    T = x.shape[0]
+    C = cq + ck + cv
+    taps = weight.shape[1]
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[1] >= C and x.is_cuda, "x must be rows of at least q + k + v channels")
+    _need(weight.shape == (C, taps) and (bias is None or bias.numel() == C), "one row of taps (and one bias) per channel")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] >= (taps - 1) * C, "the state must be float32 [slots, >= (taps - 1) * channels]")
+    rows.check(T)
+    _need(out_q.dtype == x.dtype and out_k.dtype == x.dtype and out_v.dtype == x.dtype, "results have the type of x")
+    _need(out_q.numel() >= T * cq, "out_q too small")
+    page_size = 0
+    if slots is not None:
+        _is_i32(slots, T)
+        page_size = out_k.shape[2]
+        _need(out_k.dim() == 4 and out_k.shape[1] * d == ck and out_k.shape[3] == d, "key cache must be [pages, k heads, page, head_dim]")
+        _need(out_v.shape == (out_k.shape[0], cv // vd, vd, page_size), "value cache must be [pages, v heads, value_dim, page]")
+    else:
+        _need(out_k.numel() >= T * ck and out_v.numel() >= T * cv, "out_k or out_v too small")
+    rot = 0
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.shape[0] == T and cos_sin.shape[2] == 2,
+              "the rotation table must be float32 [T, pairs, 2]")
+        rot = 2 * cos_sin.shape[1]
+    _call("ix_short_conv", x.data_ptr(), _i32(_dt(x)), _i64(x.stride(0)), _ptr(bias),
+          _i32(_dt(bias) if bias is not None else F32), _ptr(weight), _i32(_dt(weight)), _i32(taps), state.data_ptr(),
+          _i64(state.stride(0)), _ptr(rows.seq_of_token), _ptr(rows.q_start), _ptr(rows.state_slots), _ptr(cos_sin),
+          _i32(rot), _i32(1 if silu else 0), _ptr(slots), _i32(page_size), _ptr(out_q), _ptr(out_k), _ptr(out_v),
+          _i64(T), _i32(cq), _i32(ck), _i32(cv), _i32(d), _i32(vd), _stream())
+
+
+def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ab: torch.Tensor, a_log: torch.Tensor,
+               dt_bias: torch.Tensor, state: torch.Tensor, rows: StepRows, out: torch.Tensor, heads: int,
+               kv_heads: int, dim: int, vdim: int) -> None:
+    """The gated delta rule over the rows of a step, request by request, from and to `state` (a float32 view
+    [slots, >= heads * dim * vdim]).  q, k [T, kv_heads * dim], v [T, heads * vdim] (rows may be strided);
+    ab float32 [T, 2 heads]: the decay's and the step size's logits; out float32 [T, heads, vdim]."""
+    T = q.shape[0]
+    for t, n in ((q, kv_heads * dim), (k, kv_heads * dim), (v, heads * vdim)):
+        _need(t.dim() == 2 and t.shape == (T, n) and t.stride(1) == 1 and t.dtype == q.dtype and t.is_cuda, "q, k or v shape")
+    _need(ab.dtype == torch.float32 and ab.shape == (T, 2 * heads) and ab.is_contiguous(), "ab must be float32 [T, 2 heads]")
+    _need(a_log.dtype == torch.float32 and a_log.numel() == heads and dt_bias.dtype == torch.float32
+          and dt_bias.numel() == heads, "a_log and dt_bias must be float32 [heads]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] >= heads * dim * vdim, "the state must be float32 [slots, >= heads * dim * vdim]")
+    _need(out.dtype == torch.float32 and out.shape == (T, heads, vdim), "out must be float32 [T, heads, vdim]")
+    rows.check(T)
+    S = rows.q_start.numel() - 1
+    _call("ix_delta_rule", q.data_ptr(), k.data_ptr(), v.data_ptr(), _i32(_dt(q)), _i64(q.stride(0)), _i64(k.stride(0)),
+          _i64(v.stride(0)), _ptr(ab), _ptr(a_log), _ptr(dt_bias), state.data_ptr(), _i64(state.stride(0)),
+          _ptr(rows.q_start), _ptr(rows.state_slots), _ptr(out), _i64(T), _i32(S), _i32(heads), _i32(kv_heads),
+          _i32(dim), _i32(vdim), _stream())
+
+
+def head_norm_gate(x: torch.Tensor, out: torch.Tensor, eps: float, weight: Optional[torch.Tensor] = None,
+                   gate: Optional[torch.Tensor] = None, x2: Optional[torch.Tensor] = None, lam: float = 0.0,
+                   mult: float = 1.0) -> None:
+    """Per (token, head): o = x - lam * x2 (x2 optional); out = o / sqrt(mean(o^2) + eps) * weight * silu(gate) * mult.
+    x, x2 float32 [T, heads, vdim]; weight [vdim]; gate [T, >= heads * vdim] (rows may be strided) and out
+    [T, heads * vdim] of the run's type."""
+    T, heads, vdim = x.shape
+    _need(x.dtype == torch.float32 and (x2 is None or (x2.dtype == torch.float32 and x2.shape == x.shape)), "x, x2 float32")
+    _need(out.shape == (T, heads * vdim), "out must be [T, heads * vdim]")
+    _need(weight is None or weight.numel() == vdim, "one weight per value column")
+    stride = 0
+    if gate is not None:
+        _need(gate.dim() == 2 and gate.shape == (T, heads * vdim) and gate.stride(1) == 1 and gate.dtype == out.dtype
+              and gate.is_cuda, "gate must be rows of heads * vdim of out's type")
+        stride = gate.stride(0)
+    _call("ix_head_norm_gate", _ptr(x), _ptr(x2), _f32(lam), _ptr(weight), _i32(_dt(weight) if weight is not None else F32),
+          gate.data_ptr() if gate is not None else None, _i64(stride), _ptr(out), _i32(_dt(out)), _i64(T), _i32(heads),
+          _i32(vdim), _f32(eps), _f32(mult), _stream())
+
+
+def attention_diff_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                         seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, scale: float,
+                         window: int, keep_first: int, lam: float, eps: float, mult: float) -> None:
+    """Differential attention, one workgroup per (token, head): q [T, heads, 2, d], keys [pages, 2 kv_heads, page, d],
+    values [pages, kv_heads, vd, page], out [T, heads, vd] = rmsnorm(a_0 - lam a_1) * mult."""
+    T, heads, two, d = q.shape
+    _need(two == 2 and q.is_contiguous(), "q must be [T, heads, 2, d]")
+    _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and out.dtype == q.dtype, "dtype mismatch")
+    _need(k_cache.dim() == 4 and k_cache.shape[3] == d and k_cache.shape[1] % 2 == 0, "key cache must be [pages, 2 kv_heads, page, d]")
+    kv_heads, page_size = k_cache.shape[1] // 2, k_cache.shape[2]
+    _need(v_cache.dim() == 4 and v_cache.shape[0] == k_cache.shape[0] and v_cache.shape[1] == kv_heads
+          and v_cache.shape[3] == page_size, "value cache must be [pages, kv_heads, vd, page]")
+    vd = v_cache.shape[2]
+    _need(out.shape == (T, heads, vd), "out must be [T, heads, vd]")
+    _need(block_table.dim() == 2, "block table must be [requests, pages]")
+    _is_i32(block_table)
+    _is_i32(seq_of_token, T)
+    _is_i32(positions, T)
+    _call("ix_attention_diff_plain", _ptr(q), _ptr(k_cache), _ptr(v_cache), _i32(_dt(q)), _ptr(block_table),
+          _ptr(seq_of_token), _ptr(positions), _ptr(out), _i64(T), _i32(heads), _i32(kv_heads), _i32(d), _i32(vd),
+          _i32(page_size), _i32(block_table.shape[1]), _f32(scale), _i32(window), _i32(keep_first), _f32(lam),
+          _f32(eps), _f32(mult), _stream())

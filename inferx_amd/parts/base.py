@@ -60,10 +60,12 @@ class CacheNeed:
     """What a part keeps per token, in pages: the arrays it names, for all earlier tokens (`window` 0) or only
     the last W (the query's own included), so that older pages may be given back.  Parts with equal needs share a
     group of pages (one pool, one block table per request); the runner allocates each array from this description
-    and knows nothing else about it."""
+    and knows nothing else about it.  `keep_first`: with a window, the request's first `keep_first` tokens stay
+    readable as well (their pages are never given back)."""
 
     arrays: Tuple[CacheArray, ...]
     window: int = 0
+    keep_first: int = 0
 
     @staticmethod
     def keys_and_values(kv_heads: int, head_dim: int, window: int = 0, value_dim: Optional[int] = None) -> "CacheNeed":

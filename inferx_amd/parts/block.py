@@ -10,6 +10,7 @@ says so gets norm2 unapplied (`LazyNorm`) and applies it in its first kernel.
 from __future__ import annotations
 
 from .base import Block, LazyNorm, register_part, resolve_delta
+from .norm import NormedDelta
 
 
 class PreNormBlock(Block):
@@ -70,5 +71,35 @@ class GainedPreNormBlock(Block):
         return f
 
 
+class SandwichNormBlock(Block):
+    """A norm before and after each branch:
+
+        h += post1(mixer(norm1(h)));   h += post2(feed_forward(norm2(h)))
+
+    The normalised branch results travel as `NormedDelta`s, so that an RMS norm that follows (the layer's next one,
+    the next layer's first, the model's last) forms them, adds them and normalises in one kernel.  The feed-forward
+    and its two norms may be left out together."""
+
+    graph_safe = True
+    part_kinds = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm", "mixer_post_norm": "norm",
+                  "feed_forward_norm": "norm", "feed_forward_post_norm": "norm"}
+    optional_parts = ("feed_forward", "feed_forward_norm", "feed_forward_post_norm")
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        present = [p is not None for p in (self.feed_forward, self.feed_forward_norm, self.feed_forward_post_norm)]
+        if any(present) != all(present):
+            raise KeyError("a feed-forward and the norms around it come together or not at all")
+
+    def forward(self, ctx, h, pending, caches):
+        x = self.mixer_norm.forward(ctx, h, pending)
+        a = NormedDelta(resolve_delta(ctx, self.mixer.forward(ctx, x, caches.get("mixer"))), self.mixer_post_norm)
+        if self.feed_forward is None:
+            return a
+        x = self.feed_forward_norm.forward(ctx, h, a)
+        return NormedDelta(resolve_delta(ctx, self.feed_forward.forward(ctx, x)), self.feed_forward_post_norm)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "sandwich_norm", SandwichNormBlock)
 register_part("block", "prenorm_gained", GainedPreNormBlock)

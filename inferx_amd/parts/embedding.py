@@ -38,8 +38,9 @@ class TokenEmbedding(Embedding):
 class LinearHead(Head):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, init_std: float = 0.02):
+    def __init__(self, vocab_size: int, hidden_size: int, init_std: float = 0.02, scale: float = 1.0):
         self.vocab_size, self.hidden_size, self.init_std = int(vocab_size), int(hidden_size), float(init_std)
+        self.scale = float(scale)  # logits = x . W^T * scale, the product in float32
         self.weight = None
 
     def param_specs(self) -> List[ParamSpec]:
@@ -49,7 +50,8 @@ class LinearHead(Head):
         self.weight = tensors["weight"].contiguous()
 
     def forward(self, ctx, x):
-        return ctx.rt.linear_f32(x, self.weight)
+        logits = ctx.rt.linear_f32(x, self.weight)
+        return logits if self.scale == 1.0 else logits.mul_(self.scale)
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)

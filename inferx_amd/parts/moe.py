@@ -7,10 +7,14 @@ weights are stacked at load: w13 [E, 2*mi, H] (gate rows, then up rows, per
 expert) and w2 [E, H, mi] (reference: moe_ffn.h:25-34; stacking pattern
 src/model/deepseek_v2.cc:515-542).  Router scores and the shared gate are
 float32 from the product on.
+
+Two options beside that: experts without a gate (`gated=False`: down(act(up x)) with act the square of relu, weights
+w13 [E, mi, H]) and a router that chooses among groups (`groups`, `groups_keep`: the experts form equal groups of
+neighbours, a group's score is its best expert's, and only experts of the best `groups_keep` groups can be chosen).
 """
 from __future__ import annotations
 
-from typing import List
+from typing import List, Optional
 
 import torch
 
@@ -48,7 +52,8 @@ class MoeFeedForward(FeedForward):
 
     def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_width: int, shared_width: int = 0,
                  shared_gated: bool = True, renormalize: bool = False, routed_scale: float = 1.0,
-                 init_std: float = 0.02):
+                 init_std: float = 0.02, gated: bool = True, activation: Optional[str] = None, groups: int = 1,
+                 groups_keep: int = 1):
         if not 0 < top_k <= num_experts:
             raise ValueError(f"top_k {top_k} must be between 1 and num_experts {num_experts}")
         if num_experts > 1024 or top_k > 32:
@@ -57,6 +62,21 @@ class MoeFeedForward(FeedForward):
         self.expert_width, self.shared_width = int(expert_width), int(shared_width)
         self.shared_gated, self.renormalize = bool(shared_gated), bool(renormalize)
         self.routed_scale, self.init_std = float(routed_scale), float(init_std)
+        self.gated = bool(gated)
+        activation = activation or ("silu" if self.gated else "relu2")
+        if (self.gated, activation) not in ((True, "silu"), (False, "relu2")):
+            raise ValueError(f"experts {'with' if self.gated else 'without'} a gate and the activation {activation!r}: "
+                             "a gate goes with silu, no gate with relu2 (the square of relu)")
+        if not self.gated and shared_width:
+            raise ValueError("a shared expert needs gated experts")
+        self.activation = activation
+        # what the first grouped product does with its sums
+        self.first_epilogue = ops.GATE_UP_SWIGLU if self.gated else ops.RELU_SQUARED
+        self.groups, self.groups_keep = int(groups), int(groups_keep)
+        if (self.groups < 1 or self.num_experts % self.groups or not 1 <= self.groups_keep <= self.groups
+                or self.top_k > self.groups_keep * (self.num_experts // self.groups) or self.groups > 64):
+            raise ValueError(f"{self.num_experts} experts in {groups} groups of which {groups_keep} are kept for "
+                             f"top_k {self.top_k}: at most 64 equal groups, and the kept ones must hold top_k experts")
         self.wide_tiles = self.hidden_size >= WIDE_TILES_WIDTH
         # pieces of the routed experts' width that the shared expert is cut into for steps of middling size, or 0
         self.shared_pieces = self.shared_width // self.expert_width if (
@@ -70,8 +90,9 @@ class MoeFeedForward(FeedForward):
         H, mi, si, s = self.hidden_size, self.expert_width, self.shared_width, self.init_std
         specs = [ParamSpec("gate.weight", (self.num_experts, H), std=s)]
         for e in range(self.num_experts):
-            specs += [ParamSpec(f"experts.{e}.gate_proj.weight", (mi, H), std=s),
-                      ParamSpec(f"experts.{e}.up_proj.weight", (mi, H), std=s),
+            if self.gated:
+                specs.append(ParamSpec(f"experts.{e}.gate_proj.weight", (mi, H), std=s))
+            specs += [ParamSpec(f"experts.{e}.up_proj.weight", (mi, H), std=s),
                       ParamSpec(f"experts.{e}.down_proj.weight", (H, mi), std=s)]
         if si > 0:
             specs += [ParamSpec("shared_expert.gate_proj.weight", (si, H), std=s),
@@ -86,10 +107,12 @@ class MoeFeedForward(FeedForward):
         self.w_router = tensors["gate.weight"].contiguous()
         parts = []
         for e in range(E):
-            parts += [tensors[f"experts.{e}.gate_proj.weight"], tensors[f"experts.{e}.up_proj.weight"]]
+            if self.gated:
+                parts.append(tensors[f"experts.{e}.gate_proj.weight"])
+            parts.append(tensors[f"experts.{e}.up_proj.weight"])
         downs = [tensors[f"experts.{e}.down_proj.weight"] for e in range(E)]
         mi, S = self.expert_width, self.shared_pieces
-        fold = S > 0 and all(t.dtype == torch.bfloat16 for t in parts + downs) and all(
+        fold = S > 0 and self.gated and all(t.dtype == torch.bfloat16 for t in parts + downs) and all(
             tensors[f"shared_expert.{n}_proj.weight"].dtype == torch.bfloat16 for n in ("gate", "up", "down"))
         if fold:  # piece c of the shared expert: its gate rows, its up rows, and the columns of the down product
             for c in range(S):
@@ -98,7 +121,7 @@ class MoeFeedForward(FeedForward):
                 downs.append(tensors["shared_expert.down_proj.weight"][:, c * mi:(c + 1) * mi])
         else:
             self.shared_pieces = S = 0
-        self.w13_all = stack_rows(parts).view(E + S, 2 * mi, self.hidden_size)
+        self.w13_all = stack_rows(parts).view(E + S, (2 if self.gated else 1) * mi, self.hidden_size)
         self.w2_all = stack_rows(downs).view(E + S, self.hidden_size, mi)
         self.w13, self.w2 = self.w13_all[:E], self.w2_all[:E]
         if self.shared_width > 0:
@@ -117,7 +140,7 @@ class MoeFeedForward(FeedForward):
         topk_e = rt.empty((T, k), torch.int32)
         gate = rt.empty((T,), torch.float32) if self.w_shared_gate is not None else None
         ops.moe_route(x, self.w_router, self.w_shared_gate, topk_w, topk_e, gate, self.renormalize, self.routed_scale,
-                      always)
+                      always, self.groups, self.groups_keep)
         return topk_w, topk_e, gate
 
     def _tile_rows(self, ctx, x) -> int:
@@ -150,14 +173,14 @@ class MoeFeedForward(FeedForward):
         act = rt.empty((A, self.expert_width))
         y = rt.empty((A, self.hidden_size))
         if tile_rows == ops.moe_tiled_rows(self.wide_tiles):  # many rows per expert: operands staged through LDS
-            ops.moe_grouped_tiled(x, w13, act, offsets, rows, tile_map, True, self.wide_tiles)
+            ops.moe_grouped_tiled(x, w13, act, offsets, rows, tile_map, self.first_epilogue, self.wide_tiles)
             ops.moe_grouped_tiled(act, w2, y, offsets, None, tile_map, False, self.wide_tiles)
         elif tile_rows:
             # few rows: the weights are the traffic, the reduction is split over a workgroup's four wavefronts
-            ops.moe_grouped_mfma(x, w13, act, offsets, rows, tile_map, tile_rows, True, 4)
+            ops.moe_grouped_mfma(x, w13, act, offsets, rows, tile_map, tile_rows, self.first_epilogue, 4)
             ops.moe_grouped_mfma(act, w2, y, offsets, None, tile_map, tile_rows, False, 4)
         else:
-            ops.moe_grouped_plain(x, w13, act, offsets, rows, gate_up=True)
+            ops.moe_grouped_plain(x, w13, act, offsets, rows, gate_up=self.first_epilogue)
             ops.moe_grouped_plain(act, w2, y, offsets, None, gate_up=False)
         return y
 
@@ -184,7 +207,7 @@ class MoeFeedForward(FeedForward):
         feed-forward with them: `norm` = (h, delta, weight, eps, x), x still to be filled.  `always`: see `route`
         (the chosen experts are then the first `top_k` columns of what is returned)."""
         rt, T, k, E = ctx.rt, x.shape[0], self.top_k, self.num_experts
-        if always or not ops.route_one_launch_fits(T, self.hidden_size, E):
+        if always or not self._routes_in_one_launch(T):
             assert norm is None
             topk_w, topk_e, gate = self.route(ctx, x, always)
             return (topk_w, topk_e, gate) + self.dispatch(ctx, topk_e, tile_rows, always)
@@ -199,6 +222,12 @@ class MoeFeedForward(FeedForward):
                                self.renormalize, self.routed_scale, offsets, rows, dest, tile_rows, tile_map, norm)
         return topk_w, topk_e, gate, offsets, rows, dest, tile_map
 
+    def _routes_in_one_launch(self, tokens: int) -> bool:
+        """Whether the router's scores, selection and grouping of this step fit the one launch for few tokens (which
+        chooses among all experts: a router that keeps only some groups goes through the separate kernels)."""
+        return self.groups_keep == self.groups and ops.route_one_launch_fits(tokens, self.hidden_size,
+                                                                             self.num_experts)
+
     takes_lazy_norm = True
 
     def forward(self, ctx, x):
@@ -206,7 +235,7 @@ class MoeFeedForward(FeedForward):
         if isinstance(x, LazyNorm):
             # a decoding step: the norm is applied by the router's kernel, which every token's row passes anyway
             rms = x.rms_operands()
-            if rms is not None and ops.route_one_launch_fits(x.h.shape[0], self.hidden_size, self.num_experts):
+            if rms is not None and self._routes_in_one_launch(x.h.shape[0]):
                 lazy, x = x, ctx.rt.empty(tuple(x.h.shape))
                 norm = (lazy.h, lazy.delta, rms[0], rms[1], x)
             else:

@@ -7,6 +7,8 @@ from __future__ import annotations
 
 from typing import List
 
+import torch
+
 from .. import ops
 from .base import LazyDelta, Norm, ParamSpec, register_part
 
@@ -38,6 +40,31 @@ class RMSNorm(Norm):
             delta = delta.materialize(ctx)
         ops.add_rmsnorm(h, delta, self.weight, out, self.eps, rows)
         return out
+
+
+class NormedDelta(LazyDelta):
+    """A branch's result that passes a norm of its own before it is added to the residual stream (layers with a
+    norm before and after each branch): norm(tensor), not formed yet.  An RMS norm that consumes it forms it, adds
+    it and normalises the sum in one kernel; anybody else gets the normalised tensor in float32."""
+
+    def __init__(self, tensor, norm: Norm):
+        self.tensor, self.norm = tensor, norm
+
+    def materialize(self, ctx):
+        zeros = torch.zeros(tuple(self.tensor.shape), dtype=torch.float32, device=self.tensor.device)
+        rms = self.norm.rms_operands()
+        if rms is None:  # some other norm: through its own forward, in the run's type
+            return self.norm.forward(ctx, zeros, self.tensor)
+        out = torch.empty_like(zeros)
+        ops.add_rmsnorm(zeros, self.tensor, rms[0], out, rms[1])
+        return out
+
+    def add_rmsnorm(self, ctx, h, weight, eps, rows, out) -> bool:
+        rms = self.norm.rms_operands()
+        if rms is None:
+            return False
+        ops.add_normed_rmsnorm(h, self.tensor, rms[0], rms[1], weight, out, eps, rows)
+        return True
 
 
 register_part("norm", "rmsnorm", RMSNorm)
