@@ -203,3 +203,27 @@ def test_random_orders_lose_nothing(seed):
         m.free(rid)
     m.check()
     assert all(p.used_pages == 0 for p in m.pools)
+
+
+def test_a_window_keeps_the_pages_of_its_first_tokens():
+    # keep_first = 6 with pages of 4: pages 0 and 1 hold kept tokens and stay; the window gives back what lies
+    # between them and itself
+    m = CacheManager([GroupLayout(5, keep_first=6)], [16], page_size=4, max_requests=1, max_seq_len=64)
+    plain = CacheManager([GroupLayout(5)], [16], page_size=4, max_requests=1, max_seq_len=64)
+    for c in (m, plain):
+        c.add("a")
+        c.reserve("a", 40)
+        c.commit("a", 40)
+    row = m.block_row("a", 0)
+    assert row[0] >= 0 and row[1] >= 0 and row[2:9] == [-1] * 7 and row[9] >= 0
+    assert plain.block_row("a", 0)[:9] == [-1] * 9
+    assert m.pools[0].used_pages == 3
+    m.reset("a")  # preemption gives the kept pages back too
+    assert m.pools[0].used_pages == 0
+    m.reserve("a", 3)
+    m.commit("a", 3)
+    m.free("a")
+    m.check()
+    assert m.pools[0].used_pages == 0
+    # a pool sized for the window and the step also has room for the kept pages
+    assert pages_for_window(8, 4, 2, 6, keep_first=6) == pages_for_window(8, 4, 2, 6) + 2 * 2
