@@ -33,6 +33,7 @@ beside the dense layers of the Qwen2-MoE architecture at equal sizes (the same w
 feed-forward width, vocabulary and layers), both through the step function, at a few sizes of real models' layers:
 
     python bench.py --workload pelalix [--sizes 2k,4k] [--layers L] [--batch B] [--prompt-len C] [--prefill-tokens N]
+    python bench.py --workload dezudra [--sizes 1k,2k] [--layers L] [--batch B] [--prompt-len C] [--prefill-tokens N]
 
 and a whole batch through the engine's loop (scheduler, portions, decode graphs as they come, sampling) at the same
 shape:
@@ -432,6 +433,122 @@ class _SpecOnly:
         return self._spec
 
 
+def _time_prefill_and_decode(args, rt, spec, vocab, gen):
+    """(seconds for a prompt of args.prefill_tokens in one step, seconds per step of args.batch requests of one token
+    each at contexts of args.prompt_len), through the step function, random weights drawn on the device."""
+    import torch
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.parts import build_model
+    from inferx_amd.weights import random_tensors
+
+    B, C, N = args.batch, args.prompt_len, args.prefill_tokens
+    model = build_model(spec)
+    weights = {k: rt.place(v) for k, v in random_tensors(model, seed=0, dtype=args.dtype, device="cuda:0").items()}
+    cap = -(-(max(C + args.warmup + args.steps + 8, N) + 16) // PAGE) * PAGE
+    runner = ModelRunner(_SpecOnly(spec), weights, rt, page_size=PAGE, num_pages=(B + 1) * cap // PAGE,
+                         max_requests=B + 1, max_seq_len=cap, model=model)
+    runner.capture_after = 1
+    toks = lambda n: torch.randint(0, vocab, (n,), generator=gen).tolist()
+    times = []
+    for _ in range(4):  # the prompt of N tokens in one step
+        runner.add_request("p")
+        prompt = toks(N)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        runner.run_entries([("p", prompt, [N - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t)
+        runner.end_request("p")
+    pre = min(times[1:])
+    for r in range(B):  # B requests with C tokens behind them, then steps of one token each
+        runner.add_request(r)
+        for at in range(0, C, 2048):
+            runner.run_entries([(r, toks(min(2048, C - at)), [])])
+    step = lambda: runner.run_entries([(r, toks(1), [0]) for r in range(B)])
+    for _ in range(max(args.warmup, 2)):
+        step()
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dec = (time.perf_counter() - t) / args.steps
+    for r in range(B):
+        runner.end_request(r)
+    del runner, weights, model
+    torch.cuda.empty_cache()
+    return pre, dec
+
+
+# Layer sizes for `--workload dezudra`: width, heads, key/value heads, head size, experts, experts per token, an
+# expert's width, vocabulary
+DEZUDRA_SIZES = {
+    "1k": dict(width=1024, heads=8, kv_heads=2, dim=128, experts=16, top=4, ff=704, vocab=32000),
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, experts=32, top=4, ff=1408, vocab=32000),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, experts=64, top=8, ff=1408, vocab=32000),
+}
+
+
+def run_dezudra(args) -> int:
+    """Prefill of one prompt and decode steps of a batch, through the step function, for the Dezudra design (layers
+    in turn: the gated delta rule, differential attention with a window of 1,024 that keeps 4 first tokens; experts
+    of squared relu chosen among 4 groups of which 2 are kept) and for the Qwen2-MoE architecture (attention with
+    rotation, gated experts, no shared expert) at equal width, heads, head size, experts and experts per token.  One
+    JSON line; per size and model milliseconds and tokens a second of both phases, and Dezudra's time over the
+    other's."""
+    import torch
+    from inferx_amd.config import config_from_dict
+    from inferx_amd.engine.runtime import Runtime
+
+    L = args.layers or 4
+    B, C, N = args.batch, args.prompt_len, args.prefill_tokens
+    rt = Runtime(args.dtype, "cuda:0")
+    gen = torch.Generator().manual_seed(1234)
+    out = {}
+
+    def specs(z):
+        mlp = {"kind": "moe", "expert": {"ff": z["ff"]},
+               "router": {"experts": z["experts"], "top": z["top"], "groups": {"count": 4, "keep": 2}}}
+        delta = {"type": "delta", "mlp": mlp,
+                 "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "conv": 4}}
+        attention = {"type": "attention", "mlp": mlp,
+                     "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"] // 2, "vdim": z["dim"],
+                               "conv": 4, "scale": (z["dim"] // 2) ** -0.5, "diff": 0.5,
+                               "rot": {"dims": z["dim"] // 2, "base": 10000.0}, "mask": {"size": 1024, "keep_first": 4}}}
+        dez = {"architecture": "Dezudra", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+               "logit_scale": 1.0, "layers": [delta if i % 2 == 0 else attention for i in range(L)]}
+        qwen = {"architectures": ["Qwen2MoeForCausalLM"], "num_hidden_layers": L, "hidden_size": z["width"],
+                "num_attention_heads": z["heads"], "num_key_value_heads": z["kv_heads"], "head_dim": z["dim"],
+                "num_experts": z["experts"], "num_experts_per_tok": z["top"], "moe_intermediate_size": z["ff"],
+                "shared_expert_intermediate_size": 0, "intermediate_size": z["ff"], "vocab_size": z["vocab"],
+                "rope_theta": 1e6, "rms_norm_eps": 1e-6, "max_position_embeddings": 0}
+        return {"dezudra": config_from_dict(dez).model_spec(), "qwen2_moe": config_from_dict(qwen).model_spec()}
+
+    for name in [n for n in args.sizes.split(",") if n]:
+        z = DEZUDRA_SIZES[name]
+        res = {}
+        for which, spec in specs(z).items():
+            log(f"{name}: {which}")
+            pre, dec = _time_prefill_and_decode(args, rt, spec, z["vocab"], gen)
+            res[which] = {"prefill_ms": round(pre * 1e3, 3), "prefill_tokens_s": round(N / pre, 1),
+                          "decode_ms": round(dec * 1e3, 3), "decode_tokens_s": round(B / dec, 1)}
+            log(f"{name}: {which}: {res[which]}")
+        res["dezudra_over_qwen2_moe"] = {
+            "prefill": round(res["dezudra"]["prefill_ms"] / res["qwen2_moe"]["prefill_ms"], 3),
+            "decode": round(res["dezudra"]["decode_ms"] / res["qwen2_moe"]["decode_ms"], 3)}
+        out[name] = dict(res, sizes=z)
+    first = out[next(iter(out))]
+    print(json.dumps({
+        "metric": f"Dezudra decode tok/s @ batch {B} ({C}-token contexts), first size", "value": first["dezudra"]["decode_tokens_s"],
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["dezudra"]["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: seeded random weights and token ids",
+        "config": {"model": "Dezudra beside Qwen2-MoE at equal sizes", "layers": L, "global_batch": B,
+                   "seq_len": C, "prefill_tokens": N, "parallelism": "single GPU", "page_size": PAGE},
+        "sizes": out}), flush=True)
+    return 0
+
+
 def run_pelalix(args) -> int:
     """Prefill of one prompt and decode steps of a batch, through the step function, for the Pelalix design and for
     the Qwen2-MoE architecture's dense layers (attention with rotation, RMS norms, the same gated feed-forward) at
@@ -472,45 +589,11 @@ def run_pelalix(args) -> int:
         return {"pelalix": config_from_dict(pel).model_spec(), "qwen2_dense": dense}
 
     def measure(spec, z):
-        model = build_model(spec)
-        weights = {k: rt.place(v) for k, v in random_tensors(model, seed=0, dtype=args.dtype, device="cuda:0").items()}
-        cap = -(-(max(C + args.warmup + args.steps + 8, N) + 16) // PAGE) * PAGE
-        runner = ModelRunner(_SpecOnly(spec), weights, rt, page_size=PAGE, num_pages=(B + 1) * cap // PAGE,
-                             max_requests=B + 1, max_seq_len=cap, model=model)
-        runner.capture_after = 1
-        toks = lambda n: torch.randint(0, z["vocab"], (n,), generator=gen).tolist()
-        times = []
-        for _ in range(4):  # the prompt of N tokens in one step
-            runner.add_request("p")
-            prompt = toks(N)
-            torch.cuda.synchronize()
-            t = time.perf_counter()
-            runner.run_entries([("p", prompt, [N - 1])])
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t)
-            runner.end_request("p")
-        pre = min(times[1:])
-        for r in range(B):  # B requests with C tokens behind them, then steps of one token each
-            runner.add_request(r)
-            for at in range(0, C, 2048):
-                runner.run_entries([(r, toks(min(2048, C - at)), [])])
-        step = lambda: runner.run_entries([(r, toks(1), [0]) for r in range(B)])
-        for _ in range(max(args.warmup, 2)):
-            step()
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        dec = (time.perf_counter() - t) / args.steps
-        for r in range(B):
-            runner.end_request(r)
+        pre, dec = _time_prefill_and_decode(args, rt, spec, z["vocab"], gen)
         W, H, G, d, ff, V = z["width"], z["heads"], z["kv_heads"], z["dim"], z["ff"], z["vocab"]
         per_token = W * (H * d + 2 * G * d) + H * d * W + 3 * W * ff
         flops = 2.0 * N * L * per_token + 2.0 * V * W + L * 2.0 * 2.0 * H * d * N * (N + 1) / 2.0
         bytes_dec = (L * per_token + V * W + L * 2 * G * d * (C + args.warmup + args.steps // 2) * B) * elt
-        del runner, weights, model
-        torch.cuda.empty_cache()
         return {"prefill_ms": round(pre * 1e3, 3), "prefill_tokens_s": round(N / pre, 1),
                 "prefill_tflops": round(flops / pre / 1e12, 1), "prefill_frac_of_peak": round(flops / pre / peak, 4),
                 "decode_ms": round(dec * 1e3, 3), "decode_tokens_s": round(B / dec, 1),
@@ -548,7 +631,7 @@ def main() -> int:
                     help="fewer layers than the configuration has (sizes of a layer are never reduced)")
     ap.add_argument("--scarce", action="store_true", help="offline: so few pages that sequences are preempted")
     ap.add_argument("--workload", default="decode",
-                    choices=["decode", "mixed", "long", "mixed-small", "offline", "portion", "pelalix"],
+                    choices=["decode", "mixed", "long", "mixed-small", "offline", "portion", "pelalix", "dezudra"],
                     help="decode, mixed-small: the Qwen1.5-MoE-A2.7B shape (decode is the default); mixed, long: the "
                          "Qwen2-57B-A14B shape")
     ap.add_argument("--batch", type=int, default=8)
@@ -560,7 +643,7 @@ def main() -> int:
     ap.add_argument("--prefill-context", type=int, default=0,
                     help="portion: tokens that the request has read before the timed portion")
     ap.add_argument("--shape", default="a27b", choices=["a27b", "57b"], help="portion: whose layer sizes")
-    ap.add_argument("--sizes", default="2k,4k", help="pelalix: which of the layer sizes " + ", ".join(PELALIX_SIZES))
+    ap.add_argument("--sizes", default="2k,4k", help="pelalix, dezudra: which of the layer sizes " + ", ".join(PELALIX_SIZES))
     ap.add_argument("--prompt-len", type=int, default=PROMPT,
                     help="tokens of every request's prompt before it decodes (the context of the decode steps)")
     args = ap.parse_args()
@@ -568,15 +651,17 @@ def main() -> int:
         print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
         return 2
     if args.steps is None:
-        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24, "offline": 0, "portion": 2, "pelalix": 32}[args.workload]
+        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24, "offline": 0, "portion": 2, "pelalix": 32, "dezudra": 32}[args.workload]
     if args.warmup is None:
-        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4, "offline": 0, "portion": 1, "pelalix": 4}[args.workload]
+        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4, "offline": 0, "portion": 1, "pelalix": 4, "dezudra": 4}[args.workload]
     if args.workload == "offline":
         return run_offline(args)
     if args.workload == "portion":
         return run_portion(args)
     if args.workload == "pelalix":
         return run_pelalix(args)
+    if args.workload == "dezudra":
+        return run_dezudra(args)
     if args.workload != "decode":
         return run_57b(args)
     if args.layers is None:

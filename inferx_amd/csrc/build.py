@@ -29,7 +29,8 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-ta
 # per source: matrix-core accumulators in ordinary vector registers, where a kernel also rescales them with vector
 # instructions between products (the compiler otherwise copies them to and from accumulation registers every time)
 FILE_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
-              "attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+              "attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+              "attention_diff_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 # the vendor's library for dense products (csrc/gemm.hip calls its C interface)
 LINK_LIBS = ["-lhipblaslt"]

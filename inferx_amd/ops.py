@@ -1054,3 +1054,40 @@ def attention_diff_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
           _ptr(seq_of_token), _ptr(positions), _ptr(out), _i64(T), _i32(heads), _i32(kv_heads), _i32(d), _i32(vd),
           _i32(page_size), _i32(block_table.shape[1]), _f32(scale), _i32(window), _i32(keep_first), _f32(lam),
           _f32(eps), _f32(mult), _stream())
+
+
+def attention_diff_mfma_fits(head_dim: int, value_dim: int, page_size: int) -> bool:
+    """Whether the matrix-core kernel of differential attention is built for these sizes."""
+    return bool(lib().ix_attention_diff_mfma_fits(int(head_dim), int(value_dim), int(page_size)))
+
+
+def attention_diff_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                        tiles: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, n_splits: int,
+                        workspace: torch.Tensor, scale: float, window: int, keep_first: int, lam: float, eps: float,
+                        mult: float, grouped: bool = False) -> None:
+    """Differential attention on the matrix cores (bfloat16), shapes as `attention_diff_plain`.  `tiles` int32
+    [3, n_tiles]: request, first token row and rows (at most 16) of every tile; the keys that a tile reads are cut into
+    `n_splits` slices; `workspace` float32 of T * heads * 2 * n_splits * (vd + 2) numbers.  `grouped`: every tile is
+    one token, and the query heads of a key/value head (at most 16) are served side by side."""
+    T, heads, two, d = q.shape
+    _need(two == 2 and q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "bfloat16 q [T, heads, 2, d]")
+    _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "cache dtype differs from q")
+    _need(k_cache.dim() == 4 and k_cache.shape[3] == d and k_cache.shape[1] % 2 == 0, "key cache must be [pages, 2 kv_heads, page, d]")
+    kv_heads, page_size = k_cache.shape[1] // 2, k_cache.shape[2]
+    _need(v_cache.dim() == 4 and v_cache.shape[0] == k_cache.shape[0] and v_cache.shape[1] == kv_heads
+          and v_cache.shape[3] == page_size, "value cache must be [pages, kv_heads, vd, page]")
+    vd = v_cache.shape[2]
+    _need(out.shape == (T, heads, vd), "out must be [T, heads, vd]")
+    _need(attention_diff_mfma_fits(d, vd, page_size), "sizes that the matrix-core kernel is not built for")
+    _need(tiles.dim() == 2 and tiles.shape[0] == 3 and tiles.is_contiguous(), "tiles must be int32 [3, n_tiles]")
+    _is_i32(tiles)
+    _is_i32(block_table)
+    _is_i32(positions, T)
+    n_tiles = tiles.shape[1]
+    parts = T * heads * 2 * n_splits
+    _need(workspace.dtype == torch.float32 and workspace.numel() >= parts * (vd + 2), "workspace too small")
+    _call("ix_attention_diff_mfma", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]), _ptr(tiles[1]),
+          _ptr(tiles[2]), _ptr(positions), _ptr(out), workspace.data_ptr(), workspace.data_ptr() + 4 * parts * vd,
+          _i64(T), _i32(n_tiles), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(vd), _i32(page_size),
+          _i32(block_table.shape[1]), _f32(scale), _i32(window), _i32(keep_first), _f32(lam), _f32(eps), _f32(mult),
+          _i32(1 if grouped else 0), _stream())

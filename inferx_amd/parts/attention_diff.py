@@ -25,6 +25,7 @@ import torch
 
 from .. import ops
 from ..config.spec import PartSpec
+from .attention import MIN_KEYS_PER_SPLIT, QUERY_TILE, WAVES_WANTED, plan_tiles
 from .base import CacheArray, CacheNeed, Mixer, ParamSpec, StateNeed, build_part, register_part
 from .dense_mlp import stack_rows
 from .short_conv import ShortConv
@@ -103,7 +104,37 @@ class DifferentialAttention(Mixer):
         self.attend(ctx, q, cache, out)
         return rt.linear(out.view(T, self.o_dim), self.w_out)
 
+    def capture_plan(self, ctx, requests: int, longest: int) -> None:
+        """The query tiles of a step of one token per request never change (tile i = request i, row i, one query);
+        the slices of the keys follow from `longest`.  (The same plan, under the same key, as plain attention's.)"""
+        key = ("attention_tiles_host", QUERY_TILE)
+        if key not in ctx.memo:
+            tiles = torch.tensor([list(range(requests)), list(range(requests)), [1] * requests], dtype=torch.int32,
+                                 device=ctx.rt.device)
+            ctx.memo[key] = (tiles, requests, longest)
+
+    def key_slices(self, units: int, longest: int) -> int:
+        """Into how many slices each tile's keys are cut: enough wavefronts for the machine, no slice shorter than
+        MIN_KEYS_PER_SPLIT, a power of two (few distinct values, few captured graphs), 64 at most."""
+        span = min(longest, self.window + self.keep_first + QUERY_TILE + 32) if self.window > 0 else longest
+        n = 1 if units >= WAVES_WANTED else max(1, min(WAVES_WANTED // max(1, units), -(-span // MIN_KEYS_PER_SPLIT), 64))
+        return 1 << (n.bit_length() - 1)
+
     def attend(self, ctx, q, cache, out) -> None:
+        """bfloat16 with heads and pages that the matrix-core kernel is built for: that kernel, in tiles of up to 16
+        queries of a request, a (head, map) pair per wavefront (a step of one token per request: the query heads of
+        a key/value head side by side); else the plain one."""
+        page_size = cache.k.shape[2]
+        if q.dtype == torch.bfloat16 and ops.attention_diff_mfma_fits(self.head_dim, self.value_dim, page_size):
+            tiles, n_tiles, longest = plan_tiles(ctx, QUERY_TILE)
+            group = self.num_heads // self.num_kv_heads
+            grouped = ctx.one_token_each and 2 <= group <= 16
+            n_splits = self.key_slices(n_tiles * 2 * (self.num_kv_heads if grouped else self.num_heads), longest)
+            work = ctx.rt.empty((q.shape[0] * self.num_heads * 2 * n_splits * (self.value_dim + 2),), torch.float32)
+            ops.attention_diff_mfma(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, out,
+                                    n_splits, work, self.scale, self.window, self.keep_first, self.lam, self.norm_eps,
+                                    1.0 - self.diff, grouped=grouped)
+            return
         ops.attention_diff_plain(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.seq_of_token, ctx.positions,
                                  out, self.scale, self.window, self.keep_first, self.lam, self.norm_eps,
                                  1.0 - self.diff)

@@ -401,3 +401,117 @@ def test_experts_chosen_among_groups(dtype, tol, tokens, E, top, groups, keep, f
     scale = float(np.abs(want).max())
     err = np.abs(f64(got) - want).max(axis=1) / scale
     assert (err[sure] <= (2e-5 if dtype == torch.float32 else 2e-2)).all(), f"weighted sum: {err[sure].max():.2e}"
+
+
+# ---- the matrix-core kernel of differential attention ----------------------------------------------------------------
+def tiles_of(portions):
+    """int32 [3, n]: request, first row, rows of tiles of up to 16 queries, for portions [(request, first row, rows)]."""
+    t = []
+    for req, row0, n in portions:
+        for a in range(0, n, 16):
+            t.append((req, row0 + a, min(16, n - a)))
+    return torch.tensor(t, dtype=torch.int32, device=DEV).t().contiguous()
+
+
+def mfma_attend(q, kc, vc, table, tiles, positions, n_splits, scale, window, keep, lam, eps, mult, grouped=False):
+    from inferx_amd import ops
+    T, H = q.shape[0], q.shape[1]
+    V = vc.shape[2]
+    out = torch.empty((T, H, V), dtype=torch.bfloat16, device=DEV)
+    work = torch.full((T * H * 2 * n_splits * (V + 2),), float("nan"), dtype=torch.float32, device=DEV)
+    ops.attention_diff_mfma(q.to(DEV), kc, vc, table, tiles, i32(positions), out, n_splits, work, scale, window, keep, lam,
+                            eps, mult, grouped=grouped)
+    return out
+
+
+@pytest.mark.parametrize("n_splits", [1, 2, 8])
+@pytest.mark.parametrize("H,G,D,V,window,keep", [(4, 2, 32, 32, 24, 3), (3, 1, 16, 48, 0, 0), (2, 2, 16, 48, 9, 0),
+                                                 (1, 1, 16, 16, 1, 2), (4, 1, 64, 96, 33, 40), (4, 2, 128, 128, 70, 5),
+                                                 (6, 3, 48, 16, 17, 35), (2, 1, 96, 64, 64, 32)])
+def test_differential_attention_on_the_matrix_cores(H, G, D, V, window, keep, n_splits):
+    """A portion of queries at the end of a context (tiles of 16 and a ragged one), a portion at its very start, and
+    single queries elsewhere, with the keys in one slice and in several."""
+    dtype = torch.bfloat16
+    L, page = 150, 16
+    k, v = rnd((L, 2 * G, D), 1, 1.0, dtype), rnd((L, G, V), 2, 1.0, dtype)
+    singles = [keep, max(window - 1, 0), window, window + keep, 70, 99]
+    positions = list(range(0, 21)) + singles + list(range(111, 150))
+    portions = [(0, 0, 21)] + [(0, 21 + i, 1) for i in range(len(singles))] + [(0, 21 + len(singles), 39)]
+    q = rnd((len(positions), H, 2, D), 3, 1.0, dtype)
+    kc, vc, table = paged(k, v, page, dtype)
+    lam, eps, mult = 0.45, 1e-5, 0.7
+    out = mfma_attend(q, kc, vc, table, tiles_of(portions), positions, n_splits, 0.3, window, keep, lam, eps, mult)
+    want = plain_diff_attention(f64(q), f64(k).reshape(L, G, 2, D), f64(v), positions, 0.3, window, keep, lam, eps, mult)
+    close(out, want, 1.5e-2, "differential attention (matrix cores)")
+
+
+@pytest.mark.parametrize("n_splits", [1, 4])
+@pytest.mark.parametrize("H,G,D,V,window,keep", [(4, 2, 32, 32, 24, 3), (16, 1, 64, 32, 0, 0), (6, 2, 16, 96, 40, 4)])
+def test_differential_attention_one_token_each_grouped(H, G, D, V, window, keep, n_splits):
+    """Three requests of unequal contexts, one token each, the query heads of a key/value head side by side."""
+    dtype = torch.bfloat16
+    page, lens = 16, [150, 37, 1]
+    ks = [rnd((n, 2 * G, D), 10 + i, 1.0, dtype) for i, n in enumerate(lens)]
+    vs = [rnd((n, G, V), 20 + i, 1.0, dtype) for i, n in enumerate(lens)]
+    pages = sum(-(-n // page) for n in lens)
+    kc = torch.full((pages + 2, 2 * G, page, D), float("nan"), dtype=dtype)
+    vc = torch.full((pages + 2, G, V, page), float("nan"), dtype=dtype)
+    order = torch.randperm(pages + 2, generator=torch.Generator().manual_seed(3)).tolist()
+    rows, at = [], 0
+    for i, n in enumerate(lens):
+        mine = order[at:at + -(-n // page)]
+        at += len(mine)
+        rows.append(mine + [-1] * (10 - len(mine)))
+        for j in range(n):
+            kc[mine[j // page], :, j % page] = ks[i][j]
+            vc[mine[j // page], :, :, j % page] = vs[i][j]
+    q = rnd((3, H, 2, D), 3, 1.0, dtype)
+    positions = [n - 1 for n in lens]
+    lam, eps, mult = 0.3, 1e-5, 0.5
+    tiles = torch.tensor([[0, 1, 2], [0, 1, 2], [1, 1, 1]], dtype=torch.int32, device=DEV)
+    out = mfma_attend(q, kc.to(DEV), vc.to(DEV), i32(rows), tiles, positions, n_splits, 0.3, window, keep, lam, eps, mult,
+                      grouped=True)
+    for i, n in enumerate(lens):
+        want = plain_diff_attention(f64(q)[i:i + 1], f64(ks[i]).reshape(n, G, 2, D), f64(vs[i]), [n - 1], 0.3, window, keep,
+                                    lam, eps, mult)
+        close(out[i:i + 1], want, 1.5e-2, f"request {i}")
+
+
+@pytest.mark.parametrize("grouped", [False, True])
+def test_one_key_stands_out_at_every_edge_on_the_matrix_cores(grouped):
+    """As the plain kernel's test: one key far above the others is found exactly where the window and the kept
+    first tokens say, also when the pages between them hold not-a-number (they may have been given back)."""
+    H, G, D, V, L, page = 2, 1, 16, 32, 1100, 16
+    window, keep = 40, 5
+    dtype = torch.bfloat16
+    k = rnd((L, 2 * G, D), 1, 0.05)
+    v = rnd((L, G, V), 2, 1.0)
+    mark = torch.zeros(D)
+    mark[7] = 1.0
+    lam, eps, mult = 0.0, 1e-6, 1.0
+    for pos in (39, 40, 41, 47, 48, 300, 1023, 1024, 1099):
+        cases = {0: True, keep - 1: True, keep: pos - keep < window, 15: pos - 15 < window, 16: pos - 16 < window,
+                 pos - window + 1: True, pos - window: pos - window < keep, pos - window - 1: pos - window - 1 < keep,
+                 pos: True, (pos // page) * page: True, (pos // page) * page - 1: pos - ((pos // page) * page - 1) < window}
+        for key, seen in cases.items():
+            if key < 0:
+                continue
+            kk, vv = k.clone(), v.clone()
+            kk[key, 0] = mark * 40.0
+            # whole pages between the kept first tokens' page and the window hold not-a-number
+            first_dead, last_dead = 2 * page, ((pos + 1 - window) // page) * page
+            if last_dead > first_dead:
+                kk[first_dead:last_dead] = float("nan")
+                vv[first_dead:last_dead] = float("nan")
+            q = torch.zeros((1, H, 2, D))
+            q[0, :, 0] = mark * 40.0
+            kc, vc, table = paged(kk.to(dtype), vv.to(dtype), page, dtype, seed=pos)
+            tiles = torch.tensor([[0], [0], [1]], dtype=torch.int32, device=DEV)
+            for n_splits in (1, 4):
+                out = mfma_attend(q.to(dtype), kc, vc, table, tiles, [pos], n_splits, 1.0, window, keep, lam, eps, mult,
+                                  grouped=grouped)
+                target = f64(v.to(dtype))[key, 0]
+                target = target / np.sqrt(np.mean(target * target) + eps)
+                err = float(np.abs(f64(out)[0, 0] - target).max())
+                assert np.isfinite(f64(out)).all(), f"query {pos}, key {key}: not-a-number read"
+                assert (err < 3e-2) == seen, f"query {pos}, key {key}, {n_splits} slices: {'not ' if seen else ''}found (error {err:.2e})"
