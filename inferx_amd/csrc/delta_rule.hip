@@ -9,7 +9,8 @@
 //
 // The columns of S are independent recurrences (column j only ever meets v[j]), so the work is spread over
 // (request, head, block of 16 value columns): one wavefront each, four lanes per column that own every fourth row
-// of it (RPL rows a lane, in registers).  A wavefront walks its request's rows of this step in order, with the
+// of it (RPL rows a lane, in registers; VEC: a quarter of the rows each, side by side, where that quarter is a multiple
+// of eight numbers and 16-byte aligned, so that a lane reads its part of q and k in 16-byte pieces).  A wavefront walks its request's rows of this step in order, with the
 // next row's operands asked for before the present row is worked; the state is read from the request's slot at the
 // start and written back at the end.  Query head h reads the q/k head h / (heads / kv_heads).
 #include "common.h"
@@ -17,7 +18,21 @@
 #define DELTA_COLS 16   // value columns per wavefront
 #define DELTA_SPLIT 4   // lanes per column
 
-template <typename T, int RPL>
+// eight consecutive numbers as floats
+__device__ __forceinline__ void delta_load8(const float* p, float (&out)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+  out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+}
+__device__ __forceinline__ void delta_load8(const bf16_t* p, float (&out)[8]) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  out[0] = __uint_as_float(a.x << 16); out[1] = __uint_as_float(a.x & 0xffff0000u);
+  out[2] = __uint_as_float(a.y << 16); out[3] = __uint_as_float(a.y & 0xffff0000u);
+  out[4] = __uint_as_float(a.z << 16); out[5] = __uint_as_float(a.z & 0xffff0000u);
+  out[6] = __uint_as_float(a.w << 16); out[7] = __uint_as_float(a.w & 0xffff0000u);
+}
+
+template <typename T, int RPL, bool VEC>
 __global__ void __launch_bounds__(64)
 delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, int64_t q_stride,
                   int64_t k_stride, int64_t v_stride, const float* __restrict__ ab, const float* __restrict__ a_log,
@@ -35,24 +50,46 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
   const int cj = live ? col : vdim - 1;  // lanes past the last column repeat it and store nothing
 
   float* sp = state + static_cast<int64_t>(state_slots[seq]) * state_stride + static_cast<int64_t>(head) * dim * vdim;
+  // the rows of this lane: VEC part * dim / 4 + r, else r * 4 + part
+  const int quarter = dim / DELTA_SPLIT;
+  auto row_of = [&](int r) { return VEC ? (r < quarter ? part * quarter + r : dim) : r * DELTA_SPLIT + part; };
   float S[RPL];
 #pragma unroll
   for (int r = 0; r < RPL; ++r) {
-    const int i = r * DELTA_SPLIT + part;
+    const int i = row_of(r);
     S[r] = i < dim ? sp[static_cast<int64_t>(i) * vdim + cj] : 0.f;
   }
   const float rate = expf(a_log[head]), bias = dt_bias[head];
   const float q_scale = 1.0f / sqrtf(static_cast<float>(dim));
 
   float kc[RPL], qc[RPL], vc, ac, bc;  // the present row's operands
-  auto fetch = [&](int64_t row, float* kk, float* qq, float& vv, float& aa, float& bb) {
+  auto fetch = [&](int64_t row, float (&kk)[RPL], float (&qq)[RPL], float& vv, float& aa, float& bb) {
     const T* qr = q + row * q_stride + kv * dim;
     const T* kr = k + row * k_stride + kv * dim;
+    if constexpr (VEC) {
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) {
-      const int i = r * DELTA_SPLIT + part;
-      kk[r] = i < dim ? ix_load(kr + i) : 0.f;
-      qq[r] = i < dim ? ix_load(qr + i) : 0.f;
+      for (int r = 0; r < RPL; r += 8) {
+        if (r < quarter) {
+          float k8[8], q8[8];
+          delta_load8(kr + part * quarter + r, k8);
+          delta_load8(qr + part * quarter + r, q8);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            kk[r + j] = k8[j];
+            qq[r + j] = q8[j];
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) kk[r + j] = qq[r + j] = 0.f;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < RPL; ++r) {
+        const int i = r * DELTA_SPLIT + part;
+        kk[r] = i < dim ? ix_load(kr + i) : 0.f;
+        qq[r] = i < dim ? ix_load(qr + i) : 0.f;
+      }
     }
     vv = ix_load(v + row * v_stride + head * vdim + cj);
     aa = ab[row * 2 * heads + head];
@@ -107,9 +144,163 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
   if (live) {
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
-      const int i = r * DELTA_SPLIT + part;
+      const int i = row_of(r);
       if (i < dim) sp[static_cast<int64_t>(i) * vdim + col] = S[r];
     }
+  }
+}
+
+// The same recurrence for requests that bring many rows (prompt portions), bfloat16, heads of a multiple of 32
+// numbers: the wavefront brings DELTA_CHUNK rows of its q/k head, its sixteen value columns and the two logits into
+// LDS at a time, all loads of a chunk in flight at once and a chunk ahead of the arithmetic (in registers while the
+// present chunk is worked), so that a row costs its arithmetic and a few LDS reads instead of a trip to memory.
+// Same sums in the same order as the kernel above in its 16-byte form.
+#define DELTA_CHUNK 32
+typedef unsigned int delta_u32x4 __attribute__((ext_vector_type(4)));
+
+template <int RPL>
+__global__ void __launch_bounds__(64)
+delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64_t q_stride, int64_t k_stride,
+                        int64_t v_stride, const float* ab, const float* __restrict__ a_log,
+                        const float* __restrict__ dt_bias, float* __restrict__ state, int64_t state_stride,
+                        const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
+                        float* __restrict__ out, int heads, int kv_heads, int dim, int vdim) {
+  constexpr int PIECES = RPL / 2;                  // 16-byte pieces of a q or k row: dim / 8 = 4 RPL / 8
+  constexpr int PER_LANE = DELTA_CHUNK * 2 * PIECES / 64;  // pieces of a chunk's q and k rows that a lane moves
+  __shared__ delta_u32x4 qk_s[DELTA_CHUNK][2][PIECES];   // [row][k, q][piece]
+  __shared__ float v_s[DELTA_CHUNK][DELTA_COLS];
+  __shared__ float ab_s[DELTA_CHUNK][2];
+  const int lane = threadIdx.x;
+  const int col0 = blockIdx.x * DELTA_COLS;
+  const int col = col0 + lane / DELTA_SPLIT, part = lane % DELTA_SPLIT;
+  const int head = blockIdx.y, seq = blockIdx.z;
+  const int kv = head / (heads / kv_heads);
+  const int64_t row0 = q_start[seq];
+  const int n = q_start[seq + 1] - static_cast<int>(row0);
+  if (n <= 0) return;
+  const bool live = col < vdim;
+  const int cj = live ? col : vdim - 1;
+  const int quarter = dim / DELTA_SPLIT;  // == RPL here (dim a multiple of 32, RPL = dim / 4)
+
+  float* sp = state + static_cast<int64_t>(state_slots[seq]) * state_stride + static_cast<int64_t>(head) * dim * vdim;
+  float S[RPL];
+#pragma unroll
+  for (int r = 0; r < RPL; ++r) S[r] = sp[static_cast<int64_t>(part * quarter + r) * vdim + cj];
+  const float rate = expf(a_log[head]), bias = dt_bias[head];
+  const float q_scale = 1.0f / sqrtf(static_cast<float>(dim));
+
+  // what a lane moves of a chunk: PER_LANE pieces of q and k rows, DELTA_CHUNK * 16 / 64 = 8 values, one logit
+  delta_u32x4 st_qk[PER_LANE];
+  float st_v[DELTA_CHUNK * DELTA_COLS / 64], st_ab;
+  auto ask = [&](int first) {  // rows first .. first + DELTA_CHUNK - 1 of the portion (rows past its end repeat the last)
+#pragma unroll
+    for (int u = 0; u < PER_LANE; ++u) {
+      const int id = u * 64 + lane;  // piece number within the chunk: [row][k, q][piece]
+      const int r = id / (2 * PIECES), which = (id / PIECES) & 1, pc = id % PIECES;
+      const int64_t row = row0 + min(first + r, n - 1);
+      const bf16_t* src = which ? q + row * q_stride + kv * dim : k + row * k_stride + kv * dim;
+      st_qk[u] = *reinterpret_cast<const delta_u32x4*>(src + 8 * pc);
+    }
+#pragma unroll
+    for (int u = 0; u < DELTA_CHUNK * DELTA_COLS / 64; ++u) {
+      const int id = u * 64 + lane;
+      const int r = id / DELTA_COLS, c = id % DELTA_COLS;
+      st_v[u] = ix_load(v + (row0 + min(first + r, n - 1)) * v_stride + head * vdim + min(col0 + c, vdim - 1));
+    }
+    {
+      const int r = lane / 2, which = lane & 1;
+      st_ab = ab[(row0 + min(first + r, n - 1)) * 2 * heads + which * heads + head];
+    }
+  };
+  auto put = [&]() {
+#pragma unroll
+    for (int u = 0; u < PER_LANE; ++u) {
+      const int id = u * 64 + lane;
+      qk_s[id / (2 * PIECES)][(id / PIECES) & 1][id % PIECES] = st_qk[u];
+    }
+#pragma unroll
+    for (int u = 0; u < DELTA_CHUNK * DELTA_COLS / 64; ++u) {
+      const int id = u * 64 + lane;
+      v_s[id / DELTA_COLS][id % DELTA_COLS] = st_v[u];
+    }
+    ab_s[lane / 2][lane & 1] = st_ab;
+  };
+  auto fetch = [&](int r, float (&kk)[RPL], float (&qq)[RPL], float& vv, float& aa, float& bb) {
+#pragma unroll
+    for (int j = 0; j < RPL / 8; ++j) {
+      const delta_u32x4 a = qk_s[r][0][part * (RPL / 8) + j], b = qk_s[r][1][part * (RPL / 8) + j];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        kk[8 * j + 2 * e] = __uint_as_float(a[e] << 16);
+        kk[8 * j + 2 * e + 1] = __uint_as_float(a[e] & 0xffff0000u);
+        qq[8 * j + 2 * e] = __uint_as_float(b[e] << 16);
+        qq[8 * j + 2 * e + 1] = __uint_as_float(b[e] & 0xffff0000u);
+      }
+    }
+    vv = v_s[r][lane / DELTA_SPLIT];
+    aa = ab_s[r][0];
+    bb = ab_s[r][1];
+  };
+
+  ask(0);
+  for (int first = 0; first < n; first += DELTA_CHUNK) {
+    __syncthreads();  // the chunk before has been read
+    put();
+    __syncthreads();
+    if (first + DELTA_CHUNK < n) ask(first + DELTA_CHUNK);  // on their way while this chunk is worked
+    __builtin_amdgcn_sched_barrier(0);
+    const int rows = min(DELTA_CHUNK, n - first);
+    float kc[RPL], qc[RPL], vc, ac, bc;
+    fetch(0, kc, qc, vc, ac, bc);
+    for (int i = 0; i < rows; ++i) {
+      float kn[RPL], qn[RPL], vn, an, bn;
+      fetch(min(i + 1, DELTA_CHUNK - 1), kn, qn, vn, an, bn);
+      float kk = 0.f, qq = 0.f;
+#pragma unroll
+      for (int r = 0; r < RPL; ++r) {
+        kk += kc[r] * kc[r];
+        qq += qc[r] * qc[r];
+      }
+      kk += ix_dpp<IX_DPP_XOR1>(kk);
+      kk += ix_dpp<IX_DPP_XOR2>(kk);
+      qq += ix_dpp<IX_DPP_XOR1>(qq);
+      qq += ix_dpp<IX_DPP_XOR2>(qq);
+      const float k_inv = 1.0f / sqrtf(kk + 1e-6f), q_inv = q_scale / sqrtf(qq + 1e-6f);
+      const float x = ac + bias;
+      const float softplus = x > 20.f ? x : log1pf(expf(x));
+      const float g = expf(-rate * softplus);
+      const float beta = 1.0f / (1.0f + expf(-bc));
+      float dot = 0.f;
+#pragma unroll
+      for (int r = 0; r < RPL; ++r) {
+        S[r] *= g;
+        dot += S[r] * (kc[r] * k_inv);
+      }
+      dot += ix_dpp<IX_DPP_XOR1>(dot);
+      dot += ix_dpp<IX_DPP_XOR2>(dot);
+      const float u = beta * (vc - dot);
+      float o = 0.f;
+#pragma unroll
+      for (int r = 0; r < RPL; ++r) {
+        S[r] += (kc[r] * k_inv) * u;
+        o += S[r] * (qc[r] * q_inv);
+      }
+      o += ix_dpp<IX_DPP_XOR1>(o);
+      o += ix_dpp<IX_DPP_XOR2>(o);
+      if (live && part == 0) out[((row0 + first + i) * heads + head) * vdim + col] = o;
+#pragma unroll
+      for (int r = 0; r < RPL; ++r) {
+        kc[r] = kn[r];
+        qc[r] = qn[r];
+      }
+      vc = vn;
+      ac = an;
+      bc = bn;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) sp[static_cast<int64_t>(part * quarter + r) * vdim + col] = S[r];
   }
 }
 
@@ -130,16 +321,34 @@ extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dt
   if (tokens == 0 || requests == 0) return 0;
   dim3 grid((vdim + DELTA_COLS - 1) / DELTA_COLS, heads, requests), block(64);
   const int rpl = (dim + DELTA_SPLIT - 1) / DELTA_SPLIT;
-#define LAUNCH(TT, RPL)                                                                                             \
-  hipLaunchKernelGGL((delta_rule_kernel<TT, RPL>), grid, block, 0, stream, (const TT*)q, (const TT*)k, (const TT*)v, \
-                     q_stride, k_stride, v_stride, ab, a_log, dt_bias, state, state_stride, q_start, state_slots, out, \
+  // 16-byte pieces: a lane's quarter of a head is a multiple of eight numbers, and rows and heads start aligned
+  const int elt = 2;
+  const bool vec = dtype == IX_BF16 && dim % (8 * DELTA_SPLIT) == 0 && (q_stride * elt) % 16 == 0 && (k_stride * elt) % 16 == 0 &&
+                   ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k)) & 15) == 0;
+#define LAUNCH(TT, RPL, VEC)                                                                                            \
+  hipLaunchKernelGGL((delta_rule_kernel<TT, RPL, VEC>), grid, block, 0, stream, (const TT*)q, (const TT*)k, (const TT*)v, \
+                     q_stride, k_stride, v_stride, ab, a_log, dt_bias, state, state_stride, q_start, state_slots, out,    \
                      heads, kv_heads, dim, vdim)
-#define PICK(TT)                      \
-  if (rpl <= 8) LAUNCH(TT, 8);        \
-  else if (rpl <= 16) LAUNCH(TT, 16); \
-  else if (rpl <= 32) LAUNCH(TT, 32); \
-  else LAUNCH(TT, 64);
-  if (dtype == IX_F32) { PICK(float) } else { PICK(bf16_t) }
+#define PICK(TT, VEC)                      \
+  if (rpl <= 8) LAUNCH(TT, 8, VEC);        \
+  else if (rpl <= 16) LAUNCH(TT, 16, VEC); \
+  else if (rpl <= 32) LAUNCH(TT, 32, VEC); \
+  else LAUNCH(TT, 64, VEC);
+  // steps that bring a request many rows: chunks through LDS (heads of 32, 64, 96 or 128 numbers)
+  if (vec && tokens >= 4 * static_cast<int64_t>(requests) && dim % 32 == 0 && dim <= 128) {
+#define CHUNKED(RPL)                                                                                                  \
+  hipLaunchKernelGGL((delta_rule_chunk_kernel<RPL>), grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k,       \
+                     (const bf16_t*)v, q_stride, k_stride, v_stride, ab, a_log, dt_bias, state, state_stride, q_start, \
+                     state_slots, out, heads, kv_heads, dim, vdim)
+    if (dim == 32) CHUNKED(8);
+    else if (dim == 64) CHUNKED(16);
+    else if (dim == 96) CHUNKED(24);
+    else CHUNKED(32);
+#undef CHUNKED
+    return ix_check_launch("ix_delta_rule");
+  }
+  // (the 16-byte form is built for bfloat16, the type whose runs are timed)
+  if (dtype == IX_F32) { PICK(float, false) } else if (vec) { PICK(bf16_t, true) } else { PICK(bf16_t, false) }
 #undef PICK
 #undef LAUNCH
   return ix_check_launch("ix_delta_rule");
