@@ -150,29 +150,49 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
   }
 }
 
-// The same recurrence for requests that bring many rows (prompt portions), bfloat16, heads of a multiple of 32
-// numbers: the wavefront brings DELTA_CHUNK rows of its q/k head, its sixteen value columns and the two logits into
-// LDS at a time, all loads of a chunk in flight at once and a chunk ahead of the arithmetic (in registers while the
-// present chunk is worked), so that a row costs its arithmetic and a few LDS reads instead of a trip to memory.
-// Same sums in the same order as the kernel above in its 16-byte form.
+// The same recurrence for requests that bring many rows (prompt portions), bfloat16, heads of 32, 64 or 128 numbers.
+// A wavefront at one wavefront per SIMD issues one vector instruction every few cycles, so what counts here is the
+// number of instructions per row, and how many wavefronts share a head:
+//   * the wavefront brings DELTA_CHUNK rows of its q/k head, its value columns and the two logits into LDS at a
+//     time, all loads of a chunk in flight at once and a chunk ahead of the arithmetic (in registers while the
+//     present chunk is worked);
+//   * on the way into LDS the rows are made unit vectors (q also times dim^(-1/2)) and the logits become the decay
+//     and the step size, once per row instead of once per lane and row;
+//   * SP lanes share a column (4, or 16 where the head is a multiple of 64 numbers: four times the wavefronts, a
+//     quarter of the rows each), RPL = dim / SP rows a lane.
+// Per row and lane that leaves four sweeps over RPL numbers and two sums over SP lanes.  (The decay is applied to
+// the product S^T k instead of to S first, which is the same number up to rounding.)
 #define DELTA_CHUNK 32
 typedef unsigned int delta_u32x4 __attribute__((ext_vector_type(4)));
+typedef float delta_f32x4 __attribute__((ext_vector_type(4)));
 
-template <int RPL>
+template <int SP>
+__device__ __forceinline__ float delta_sum_over(float x) {  // over the SP neighbouring lanes of a column
+  x += ix_dpp<IX_DPP_XOR1>(x);
+  x += ix_dpp<IX_DPP_XOR2>(x);
+  if constexpr (SP >= 8) x += ix_dpp<IX_DPP_HALF_MIRROR>(x);
+  if constexpr (SP >= 16) x += ix_dpp<IX_DPP_MIRROR>(x);
+  return x;
+}
+
+template <int SP, int RPL>
 __global__ void __launch_bounds__(64)
 delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64_t q_stride, int64_t k_stride,
                         int64_t v_stride, const float* ab, const float* __restrict__ a_log,
                         const float* __restrict__ dt_bias, float* __restrict__ state, int64_t state_stride,
                         const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
-                        float* __restrict__ out, int heads, int kv_heads, int dim, int vdim) {
-  constexpr int PIECES = RPL / 2;                  // 16-byte pieces of a q or k row: dim / 8 = 4 RPL / 8
+                        float* __restrict__ out, int heads, int kv_heads, int vdim) {
+  constexpr int DIM = SP * RPL;
+  constexpr int COLS = 64 / SP;                      // value columns of a wavefront
+  constexpr int PIECES = DIM / 8;                    // 16-byte pieces of a q or k row (4, 8 or 16: a power of two)
   constexpr int PER_LANE = DELTA_CHUNK * 2 * PIECES / 64;  // pieces of a chunk's q and k rows that a lane moves
-  __shared__ delta_u32x4 qk_s[DELTA_CHUNK][2][PIECES];   // [row][k, q][piece]
-  __shared__ float v_s[DELTA_CHUNK][DELTA_COLS];
-  __shared__ float ab_s[DELTA_CHUNK][2];
+  constexpr int V_PER_LANE = (DELTA_CHUNK * COLS + 63) / 64;
+  __shared__ delta_f32x4 qk_s[DELTA_CHUNK][2][DIM / 4];  // [row][k, q]: unit vectors (q times dim^(-1/2))
+  __shared__ float v_s[DELTA_CHUNK][COLS];
+  __shared__ float gb_s[DELTA_CHUNK][2];             // decay, step size
   const int lane = threadIdx.x;
-  const int col0 = blockIdx.x * DELTA_COLS;
-  const int col = col0 + lane / DELTA_SPLIT, part = lane % DELTA_SPLIT;
+  const int col0 = blockIdx.x * COLS;
+  const int col = col0 + lane / SP, part = lane % SP;
   const int head = blockIdx.y, seq = blockIdx.z;
   const int kv = head / (heads / kv_heads);
   const int64_t row0 = q_start[seq];
@@ -180,31 +200,29 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
   if (n <= 0) return;
   const bool live = col < vdim;
   const int cj = live ? col : vdim - 1;
-  const int quarter = dim / DELTA_SPLIT;  // == RPL here (dim a multiple of 32, RPL = dim / 4)
 
-  float* sp = state + static_cast<int64_t>(state_slots[seq]) * state_stride + static_cast<int64_t>(head) * dim * vdim;
+  float* sp = state + static_cast<int64_t>(state_slots[seq]) * state_stride + static_cast<int64_t>(head) * DIM * vdim;
   float S[RPL];
 #pragma unroll
-  for (int r = 0; r < RPL; ++r) S[r] = sp[static_cast<int64_t>(part * quarter + r) * vdim + cj];
+  for (int r = 0; r < RPL; ++r) S[r] = sp[static_cast<int64_t>(part * RPL + r) * vdim + cj];
   const float rate = expf(a_log[head]), bias = dt_bias[head];
-  const float q_scale = 1.0f / sqrtf(static_cast<float>(dim));
+  const float q_scale = 1.0f / sqrtf(static_cast<float>(DIM));
 
-  // what a lane moves of a chunk: PER_LANE pieces of q and k rows, DELTA_CHUNK * 16 / 64 = 8 values, one logit
   delta_u32x4 st_qk[PER_LANE];
-  float st_v[DELTA_CHUNK * DELTA_COLS / 64], st_ab;
+  float st_v[V_PER_LANE], st_ab;
   auto ask = [&](int first) {  // rows first .. first + DELTA_CHUNK - 1 of the portion (rows past its end repeat the last)
 #pragma unroll
     for (int u = 0; u < PER_LANE; ++u) {
       const int id = u * 64 + lane;  // piece number within the chunk: [row][k, q][piece]
       const int r = id / (2 * PIECES), which = (id / PIECES) & 1, pc = id % PIECES;
       const int64_t row = row0 + min(first + r, n - 1);
-      const bf16_t* src = which ? q + row * q_stride + kv * dim : k + row * k_stride + kv * dim;
+      const bf16_t* src = which ? q + row * q_stride + kv * DIM : k + row * k_stride + kv * DIM;
       st_qk[u] = *reinterpret_cast<const delta_u32x4*>(src + 8 * pc);
     }
 #pragma unroll
-    for (int u = 0; u < DELTA_CHUNK * DELTA_COLS / 64; ++u) {
-      const int id = u * 64 + lane;
-      const int r = id / DELTA_COLS, c = id % DELTA_COLS;
+    for (int u = 0; u < V_PER_LANE; ++u) {
+      const int id = min(u * 64 + lane, DELTA_CHUNK * COLS - 1);
+      const int r = id / COLS, c = id % COLS;
       st_v[u] = ix_load(v + (row0 + min(first + r, n - 1)) * v_stride + head * vdim + min(col0 + c, vdim - 1));
     }
     {
@@ -216,30 +234,46 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
 #pragma unroll
     for (int u = 0; u < PER_LANE; ++u) {
       const int id = u * 64 + lane;
-      qk_s[id / (2 * PIECES)][(id / PIECES) & 1][id % PIECES] = st_qk[u];
-    }
-#pragma unroll
-    for (int u = 0; u < DELTA_CHUNK * DELTA_COLS / 64; ++u) {
-      const int id = u * 64 + lane;
-      v_s[id / DELTA_COLS][id % DELTA_COLS] = st_v[u];
-    }
-    ab_s[lane / 2][lane & 1] = st_ab;
-  };
-  auto fetch = [&](int r, float (&kk)[RPL], float (&qq)[RPL], float& vv, float& aa, float& bb) {
-#pragma unroll
-    for (int j = 0; j < RPL / 8; ++j) {
-      const delta_u32x4 a = qk_s[r][0][part * (RPL / 8) + j], b = qk_s[r][1][part * (RPL / 8) + j];
+      const int r = id / (2 * PIECES), which = (id / PIECES) & 1, pc = id % PIECES;
+      float x[8];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        kk[8 * j + 2 * e] = __uint_as_float(a[e] << 16);
-        kk[8 * j + 2 * e + 1] = __uint_as_float(a[e] & 0xffff0000u);
-        qq[8 * j + 2 * e] = __uint_as_float(b[e] << 16);
-        qq[8 * j + 2 * e + 1] = __uint_as_float(b[e] & 0xffff0000u);
+        x[2 * e] = __uint_as_float(st_qk[u][e] << 16);
+        x[2 * e + 1] = __uint_as_float(st_qk[u][e] & 0xffff0000u);
+      }
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+      ss = delta_sum_over<PIECES>(ss);  // a row's pieces lie in PIECES neighbouring lanes
+      const float f = (which ? q_scale : 1.0f) / sqrtf(ss + 1e-6f);
+      qk_s[r][which][2 * pc] = delta_f32x4{x[0] * f, x[1] * f, x[2] * f, x[3] * f};
+      qk_s[r][which][2 * pc + 1] = delta_f32x4{x[4] * f, x[5] * f, x[6] * f, x[7] * f};
+    }
+#pragma unroll
+    for (int u = 0; u < V_PER_LANE; ++u) {
+      const int id = u * 64 + lane;
+      if (id < DELTA_CHUNK * COLS) v_s[id / COLS][id % COLS] = st_v[u];
+    }
+    if (lane & 1) {
+      gb_s[lane / 2][1] = 1.0f / (1.0f + expf(-st_ab));
+    } else {
+      const float x = st_ab + bias;
+      gb_s[lane / 2][0] = expf(-rate * (x > 20.f ? x : log1pf(expf(x))));
+    }
+  };
+  auto fetch = [&](int r, float (&kk)[RPL], float (&qq)[RPL], float& vv, float& gg, float& bb) {
+#pragma unroll
+    for (int j = 0; j < RPL / 4; ++j) {
+      const delta_f32x4 a = qk_s[r][0][part * (RPL / 4) + j], b = qk_s[r][1][part * (RPL / 4) + j];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        kk[4 * j + e] = a[e];
+        qq[4 * j + e] = b[e];
       }
     }
-    vv = v_s[r][lane / DELTA_SPLIT];
-    aa = ab_s[r][0];
-    bb = ab_s[r][1];
+    vv = v_s[r][lane / SP];
+    gg = gb_s[r][0];
+    bb = gb_s[r][1];
   };
 
   ask(0);
@@ -250,43 +284,23 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
     if (first + DELTA_CHUNK < n) ask(first + DELTA_CHUNK);  // on their way while this chunk is worked
     __builtin_amdgcn_sched_barrier(0);
     const int rows = min(DELTA_CHUNK, n - first);
-    float kc[RPL], qc[RPL], vc, ac, bc;
-    fetch(0, kc, qc, vc, ac, bc);
+    float kc[RPL], qc[RPL], vc, gc, bc;
+    fetch(0, kc, qc, vc, gc, bc);
     for (int i = 0; i < rows; ++i) {
-      float kn[RPL], qn[RPL], vn, an, bn;
-      fetch(min(i + 1, DELTA_CHUNK - 1), kn, qn, vn, an, bn);
-      float kk = 0.f, qq = 0.f;
-#pragma unroll
-      for (int r = 0; r < RPL; ++r) {
-        kk += kc[r] * kc[r];
-        qq += qc[r] * qc[r];
-      }
-      kk += ix_dpp<IX_DPP_XOR1>(kk);
-      kk += ix_dpp<IX_DPP_XOR2>(kk);
-      qq += ix_dpp<IX_DPP_XOR1>(qq);
-      qq += ix_dpp<IX_DPP_XOR2>(qq);
-      const float k_inv = 1.0f / sqrtf(kk + 1e-6f), q_inv = q_scale / sqrtf(qq + 1e-6f);
-      const float x = ac + bias;
-      const float softplus = x > 20.f ? x : log1pf(expf(x));
-      const float g = expf(-rate * softplus);
-      const float beta = 1.0f / (1.0f + expf(-bc));
+      float kn[RPL], qn[RPL], vn, gn, bn;
+      fetch(min(i + 1, DELTA_CHUNK - 1), kn, qn, vn, gn, bn);
       float dot = 0.f;
 #pragma unroll
-      for (int r = 0; r < RPL; ++r) {
-        S[r] *= g;
-        dot += S[r] * (kc[r] * k_inv);
-      }
-      dot += ix_dpp<IX_DPP_XOR1>(dot);
-      dot += ix_dpp<IX_DPP_XOR2>(dot);
-      const float u = beta * (vc - dot);
+      for (int r = 0; r < RPL; ++r) dot += S[r] * kc[r];
+      dot = delta_sum_over<SP>(dot);
+      const float u = bc * (vc - gc * dot);
       float o = 0.f;
 #pragma unroll
       for (int r = 0; r < RPL; ++r) {
-        S[r] += (kc[r] * k_inv) * u;
-        o += S[r] * (qc[r] * q_inv);
+        S[r] = fmaf(S[r], gc, kc[r] * u);
+        o += S[r] * qc[r];
       }
-      o += ix_dpp<IX_DPP_XOR1>(o);
-      o += ix_dpp<IX_DPP_XOR2>(o);
+      o = delta_sum_over<SP>(o);
       if (live && part == 0) out[((row0 + first + i) * heads + head) * vdim + col] = o;
 #pragma unroll
       for (int r = 0; r < RPL; ++r) {
@@ -294,13 +308,13 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
         qc[r] = qn[r];
       }
       vc = vn;
-      ac = an;
+      gc = gn;
       bc = bn;
     }
   }
   if (live) {
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) sp[static_cast<int64_t>(part * quarter + r) * vdim + col] = S[r];
+    for (int r = 0; r < RPL; ++r) sp[static_cast<int64_t>(part * RPL + r) * vdim + col] = S[r];
   }
 }
 
@@ -334,16 +348,15 @@ extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dt
   else if (rpl <= 16) LAUNCH(TT, 16, VEC); \
   else if (rpl <= 32) LAUNCH(TT, 32, VEC); \
   else LAUNCH(TT, 64, VEC);
-  // steps that bring a request many rows: chunks through LDS (heads of 32, 64, 96 or 128 numbers)
-  if (vec && tokens >= 4 * static_cast<int64_t>(requests) && dim % 32 == 0 && dim <= 128) {
-#define CHUNKED(RPL)                                                                                                  \
-  hipLaunchKernelGGL((delta_rule_chunk_kernel<RPL>), grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k,       \
-                     (const bf16_t*)v, q_stride, k_stride, v_stride, ab, a_log, dt_bias, state, state_stride, q_start, \
-                     state_slots, out, heads, kv_heads, dim, vdim)
-    if (dim == 32) CHUNKED(8);
-    else if (dim == 64) CHUNKED(16);
-    else if (dim == 96) CHUNKED(24);
-    else CHUNKED(32);
+  // steps that bring a request many rows: chunks through LDS (heads of 32, 64 or 128 numbers)
+  if (vec && tokens >= 4 * static_cast<int64_t>(requests) && (dim == 32 || dim == 64 || dim == 128)) {
+#define CHUNKED(SP, RPL)                                                                                                  \
+  hipLaunchKernelGGL((delta_rule_chunk_kernel<SP, RPL>), dim3((vdim + 64 / SP - 1) / (64 / SP), heads, requests), block, 0, \
+                     stream, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, q_stride, k_stride, v_stride, ab, a_log, \
+                     dt_bias, state, state_stride, q_start, state_slots, out, heads, kv_heads, vdim)
+    if (dim == 32) CHUNKED(4, 8);
+    else if (dim == 64) CHUNKED(16, 4);
+    else CHUNKED(16, 8);
 #undef CHUNKED
     return ix_check_launch("ix_delta_rule");
   }
