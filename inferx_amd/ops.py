@@ -951,13 +951,16 @@ class StepRows:
 def short_conv(x: torch.Tensor, bias: Optional[torch.Tensor], weight: torch.Tensor, state: torch.Tensor,
                rows: StepRows, sizes: Tuple[int, int, int, int, int], out_q: torch.Tensor,
                out_k: torch.Tensor, out_v: torch.Tensor, slots: Optional[torch.Tensor] = None,
-               cos_sin: Optional[torch.Tensor] = None, silu: bool = False) -> None:
+               cos_sin: Optional[torch.Tensor] = None, silu: bool = False, weight_t: Optional[torch.Tensor] = None,
+               bias_f32: Optional[torch.Tensor] = None) -> None:
     """A causal convolution of `taps` = weight.shape[1] taps over time on the first q + k + v channels of x
     [T, >= channels] (a bias added first), continued from `state` (a float32 view [slots, >= (taps - 1) * channels]
     of each request's last inputs, brought up to date), then silu and / or the rotation of the first
     2 * cos_sin.shape[1] elements of every q and k head.  `sizes` = (q channels, k channels, v channels, head_dim,
     value_dim).  With `slots` k and v go into the paged caches out_k [pages, k heads, page, head_dim] and out_v
-    [pages, v heads, value_dim, page]; else to rows [T, k channels], [T, v channels].  q goes to out_q [T, q channels]."""
+    [pages, v heads, value_dim, page]; else to rows [T, k channels], [T, v channels].  q goes to out_q [T, q channels].
+    `weight_t` float32 [taps, channels] and `bias_f32` float32 [channels]: the same numbers as `weight` and `bias`, laid
+    out for the kernel's 16-byte form (used where the sizes come in eights)."""
     cq, ck, cv, d, vd = sizes
     T = x.shape[0]
     C = cq + ck + cv
@@ -982,11 +985,15 @@ def short_conv(x: torch.Tensor, bias: Optional[torch.Tensor], weight: torch.Tens
         _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.shape[0] == T and cos_sin.shape[2] == 2,
               "the rotation table must be float32 [T, pairs, 2]")
         rot = 2 * cos_sin.shape[1]
+    if weight_t is not None:
+        _need(weight_t.dtype == torch.float32 and weight_t.shape == (taps, C) and weight_t.is_contiguous(), "weight_t shape")
+    if bias_f32 is not None:
+        _need(bias_f32.dtype == torch.float32 and bias_f32.numel() == C and bias_f32.is_contiguous(), "bias_f32 shape")
     _call("ix_short_conv", x.data_ptr(), _i32(_dt(x)), _i64(x.stride(0)), _ptr(bias),
           _i32(_dt(bias) if bias is not None else F32), _ptr(weight), _i32(_dt(weight)), _i32(taps), state.data_ptr(),
           _i64(state.stride(0)), _ptr(rows.seq_of_token), _ptr(rows.q_start), _ptr(rows.state_slots), _ptr(cos_sin),
           _i32(rot), _i32(1 if silu else 0), _ptr(slots), _i32(page_size), _ptr(out_q), _ptr(out_k), _ptr(out_v),
-          _i64(T), _i32(cq), _i32(ck), _i32(cv), _i32(d), _i32(vd), _stream())
+          _i64(T), _i32(cq), _i32(ck), _i32(cv), _i32(d), _i32(vd), _ptr(weight_t), _ptr(bias_f32), _stream())
 
 
 def delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ab: torch.Tensor, a_log: torch.Tensor,

@@ -101,26 +101,30 @@ def test_normed_branch_add_and_norm(dtype, tol, width):
 
 
 # ---- the short convolution over steps, with silu, with rotation, into pages --------------------------------------
+@pytest.mark.parametrize("eights", [False, True])
 @pytest.mark.parametrize("taps", [1, 2, 4, 7])
 @pytest.mark.parametrize("dtype,tol", TYPES)
-def test_short_convolution_over_steps(dtype, tol, taps):
+def test_short_convolution_over_steps(dtype, tol, taps, eights):
     """Whatever the cut, row t reads the rows t - taps + 1 .. t of its own sequence and zeros before its start; the
     state starts as not-a-number and is cleared when a request starts."""
     from inferx_amd import ops
-    sizes = (2 * 12, 12, 3 * 20, 12, 20)  # q: two heads of 12, k: one, v: three of 20
+    # q: two heads of 12, k: one, v: three of 20; or everything in eights (the kernel's 16-byte form in bfloat16)
+    sizes = (2 * 16, 16, 3 * 24, 16, 24) if eights else (2 * 12, 12, 3 * 20, 12, 20)
     C = sizes[0] + sizes[1] + sizes[2]
-    extra = 5  # the projection's rows are wider than the convolved channels
+    extra = 8 if eights else 5  # the projection's rows are wider than the convolved channels
     w = rnd((C, taps), 3, 0.5, dtype)
     bias = rnd((C,), 4, 0.5, dtype)
     xs = [rnd((n, C + extra), 10 + r, 1.0, dtype) for r, n in enumerate(LENGTHS)]
-    state = torch.full((2, max(1, (taps - 1) * C) + 3), float("nan"), device=DEV)
+    state = torch.full((2, max(1, (taps - 1) * C) + (4 if eights else 3)), float("nan"), device=DEV)
     want = {r: pd.silu(pd.short_conv(f64(xs[r])[:, :C] + f64(bias), f64(w))) for r in range(3)}
+    fast = dict(weight_t=w.to(DEV).float().t().contiguous(), bias_f32=bias.to(DEV).float()) if eights else {}
 
     def run_step(parts, seq, pos, q_start, slots):
         x = torch.cat([xs[r][a:a + n] for r, a, n in parts]).to(DEV)
         T = x.shape[0]
         q, k, v = (torch.empty((T, c), dtype=dtype, device=DEV) for c in sizes[:3])
-        ops.short_conv(x, bias.to(DEV), w.to(DEV), state, ops.StepRows(seq, q_start, slots), sizes, q, k, v, silu=True)
+        ops.short_conv(x, bias.to(DEV), w.to(DEV), state, ops.StepRows(seq, q_start, slots), sizes, q, k, v, silu=True,
+                       **fast)
         return torch.cat([q, k, v], dim=1).cpu()
 
     got = run_in_steps(run_step, [state])
@@ -128,14 +132,14 @@ def test_short_convolution_over_steps(dtype, tol, taps):
         close(got[r], want[r], tol, f"request {r}, {taps} taps")
 
 
-@pytest.mark.parametrize("rot", [0, 4, 12])
+@pytest.mark.parametrize("D,V,rot", [(12, 20, 0), (12, 20, 4), (12, 20, 12), (16, 24, 0), (32, 8, 16), (32, 40, 32)])
 @pytest.mark.parametrize("dtype,tol", TYPES)
-def test_short_convolution_rotates_and_appends(dtype, tol, rot):
+def test_short_convolution_rotates_and_appends(dtype, tol, D, V, rot):
     """The convolved keys and values land in the request's pages (keys rotated, values transposed within a page),
     the queries in rows; pairs (i, i + rot / 2) of every head's first `rot` elements are rotated by the position."""
     from inferx_amd import ops
-    D, V, page = 12, 20, 4
-    sizes = (2 * D, 2 * D, V, D, V)
+    page = 4
+    sizes = (2 * D, 2 * D, V, D, V)  # (sizes in eights go through the kernel's 16-byte form in bfloat16)
     C, taps = sizes[0] + sizes[1] + sizes[2], 3
     w = rnd((C, taps), 3, 0.5, dtype)
     xs = [rnd((n, C), 20 + r, 1.0, dtype) for r, n in enumerate(LENGTHS)]
@@ -162,7 +166,7 @@ def test_short_convolution_rotates_and_appends(dtype, tol, rot):
             ops.rope_table(table, pos, inv_freq)
         q = torch.empty((T, 2 * D), dtype=dtype, device=DEV)
         ops.short_conv(x, None, w.to(DEV), state, ops.StepRows(seq, q_start, slots), sizes, q, k_cache, v_cache,
-                       slots=where, cos_sin=table)
+                       slots=where, cos_sin=table, weight_t=w.to(DEV).float().t().contiguous())
         # read this step's keys and values back from the pages
         flat = where.long()
         k = k_cache.permute(0, 2, 1, 3).reshape(-1, 2 * D)[flat]
