@@ -237,12 +237,14 @@ attn_diff_combine_kernel(const float* __restrict__ part_o, const float* __restri
     const float inv_l = 1.0f / ix_wave_sum(w * l_s);
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) a[mp][jj] = 0.f;
+    // (columns past the head's end read its last column again: every load is unconditional, so that the loads of
+    // several slices are in flight together; what they sum is dropped below)
+#pragma unroll 4
     for (int s = 0; s < n_splits; ++s) {
       const float ws = __shfl(w, s, 64);
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
-        const int j = lane + 64 * jj;
-        if (j < value_dim) a[mp][jj] += ws * part_o[(p0 + s) * value_dim + j];
+        if (64 * jj < value_dim) a[mp][jj] += ws * part_o[(p0 + s) * value_dim + min(lane + 64 * jj, value_dim - 1)];
       }
     }
 #pragma unroll

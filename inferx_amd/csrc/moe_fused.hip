@@ -5,6 +5,8 @@
 // Arithmetic and order of additions are those of ix_moe_combine followed by
 // ix_add_rmsnorm, except that the feed-forward's sum is not rounded to the
 // activations' type before it joins the float32 residual stream.
+// With `wd` the feed-forward's sum passes an RMS norm of its own first (layers that norm a branch's result as well):
+//   f = sum ...;  v = h[row] + f * rsqrt(mean(f^2) + eps_d) * wd
 #include "common.h"
 
 template <typename T>
@@ -12,7 +14,8 @@ __global__ void moe_combine_add_rmsnorm_kernel(float* __restrict__ h, const T* _
                                                const int32_t* __restrict__ dest, const float* __restrict__ topk_w,
                                                const T* __restrict__ shared, const float* __restrict__ shared_gate,
                                                const void* __restrict__ w, int w_dtype, T* __restrict__ out,
-                                               const int32_t* __restrict__ rows, int64_t width, int k, float eps) {
+                                               const int32_t* __restrict__ rows, int64_t width, int k, float eps,
+                                               const void* __restrict__ wd, int wd_dtype, float eps_d) {
   extern __shared__ __align__(16) float vrow[];  // [width]
   __shared__ float red[16];
   __shared__ float sw[32];
@@ -27,14 +30,33 @@ __global__ void moe_combine_add_rmsnorm_kernel(float* __restrict__ h, const T* _
   const float sg = shared ? (shared_gate ? shared_gate[row] : 1.0f) : 0.f;
   float* hr = h + row * width;
   float sumsq = 0.f;
-  for (int64_t c = threadIdx.x; c < width; c += blockDim.x) {
-    float acc = 0.f;
-    for (int s = 0; s < k; ++s) acc += sw[s] * ix_load(y + static_cast<int64_t>(sd[s]) * width + c);
-    if (shared) acc += sg * ix_load(shared + row * width + c);
-    const float v = hr[c] + acc;
-    if (!rows) hr[c] = v;
-    vrow[c] = v;
-    sumsq += v * v;
+  if (wd) {  // the sum is normalised before it is added
+    float sumsq_d = 0.f;
+    for (int64_t c = threadIdx.x; c < width; c += blockDim.x) {
+      float acc = 0.f;
+      for (int s = 0; s < k; ++s) acc += sw[s] * ix_load(y + static_cast<int64_t>(sd[s]) * width + c);
+      if (shared) acc += sg * ix_load(shared + row * width + c);
+      vrow[c] = acc;
+      sumsq_d += acc * acc;
+    }
+    sumsq_d = ix_block_sum(sumsq_d, red);
+    const float inv_d = 1.0f / sqrtf(sumsq_d / static_cast<float>(width) + eps_d);
+    for (int64_t c = threadIdx.x; c < width; c += blockDim.x) {  // (every thread reads back what it wrote itself)
+      const float v = hr[c] + vrow[c] * inv_d * ix_load_rt(wd, wd_dtype, c);
+      if (!rows) hr[c] = v;
+      vrow[c] = v;
+      sumsq += v * v;
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < width; c += blockDim.x) {
+      float acc = 0.f;
+      for (int s = 0; s < k; ++s) acc += sw[s] * ix_load(y + static_cast<int64_t>(sd[s]) * width + c);
+      if (shared) acc += sg * ix_load(shared + row * width + c);
+      const float v = hr[c] + acc;
+      if (!rows) hr[c] = v;
+      vrow[c] = v;
+      sumsq += v * v;
+    }
   }
   sumsq = ix_block_sum(sumsq, red);
   const float inv = 1.0f / sqrtf(sumsq / static_cast<float>(width) + eps);
@@ -110,7 +132,8 @@ __global__ void moe_combine_add_rmsnorm_vec4_kernel(float* __restrict__ h, const
 extern "C" int ix_moe_combine_add_rmsnorm(void* h, const void* y, int dtype, const int32_t* dest,
                                           const float* topk_w, const void* shared, const float* shared_gate,
                                           const void* w, int w_dtype, void* out, const int32_t* rows,
-                                          int64_t n_out_rows, int64_t width, int k, float eps, hipStream_t stream) {
+                                          int64_t n_out_rows, int64_t width, int k, float eps, const void* wd,
+                                          int wd_dtype, float eps_d, hipStream_t stream) {
   IX_REQUIRE(n_out_rows >= 0 && width > 0, "sizes must be positive");
   IX_REQUIRE(k > 0 && k <= 32, "top_k must be between 1 and 32");
   IX_REQUIRE(width * sizeof(float) <= 60 * 1024, "hidden width too large for the fused kernel (limit 15360)");
@@ -120,8 +143,9 @@ extern "C" int ix_moe_combine_add_rmsnorm(void* h, const void* y, int dtype, con
   const size_t smem = width * sizeof(float);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(moe_combine_add_rmsnorm_kernel<float>, grid, block, smem, stream, (float*)h, (const float*)y,
-                       dest, topk_w, (const float*)shared, shared_gate, w, w_dtype, (float*)out, rows, width, k, eps);
-  else if (dtype == IX_BF16 && width % 4 == 0 &&
+                       dest, topk_w, (const float*)shared, shared_gate, w, w_dtype, (float*)out, rows, width, k, eps, wd,
+                       wd_dtype, eps_d);
+  else if (dtype == IX_BF16 && wd == nullptr && width % 4 == 0 &&
            ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(shared) |
              reinterpret_cast<uintptr_t>(out)) & 15) == 0)
     hipLaunchKernelGGL(moe_combine_add_rmsnorm_vec4_kernel, grid, dim3(width >= 4096 ? 1024 : (width >= 2048 ? 512 : 256)),
@@ -130,7 +154,7 @@ extern "C" int ix_moe_combine_add_rmsnorm(void* h, const void* y, int dtype, con
   else if (dtype == IX_BF16)
     hipLaunchKernelGGL(moe_combine_add_rmsnorm_kernel<bf16_t>, grid, block, smem, stream, (float*)h,
                        (const bf16_t*)y, dest, topk_w, (const bf16_t*)shared, shared_gate, w, w_dtype, (bf16_t*)out,
-                       rows, width, k, eps);
+                       rows, width, k, eps, wd, wd_dtype, eps_d);
   else
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_moe_combine_add_rmsnorm");

@@ -93,11 +93,11 @@ class SandwichNormBlock(Block):
 
     def forward(self, ctx, h, pending, caches):
         x = self.mixer_norm.forward(ctx, h, pending)
-        a = NormedDelta(resolve_delta(ctx, self.mixer.forward(ctx, x, caches.get("mixer"))), self.mixer_post_norm)
+        a = NormedDelta(self.mixer.forward(ctx, x, caches.get("mixer")), self.mixer_post_norm)
         if self.feed_forward is None:
             return a
         x = self.feed_forward_norm.forward(ctx, h, a)
-        return NormedDelta(resolve_delta(ctx, self.feed_forward.forward(ctx, x)), self.feed_forward_post_norm)
+        return NormedDelta(self.feed_forward.forward(ctx, x), self.feed_forward_post_norm)
 
 
 register_part("block", "prenorm", PreNormBlock)

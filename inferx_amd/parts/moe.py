@@ -284,5 +284,13 @@ class MoeSum(LazyDelta):
         ops.moe_combine_add_rmsnorm(h, self.y, self.dest, self.topk_w, self.shared, self.gate, weight, out, eps, rows)
         return True
 
+    def add_normed_rmsnorm(self, ctx, h, sum_weight, sum_eps, weight, eps, rows, out) -> bool:
+        """As `add_rmsnorm`, with the sum passing an RMS norm of its own before it is added."""
+        if self.width * 4 > 60 * 1024 or out is None:
+            return False
+        ops.moe_combine_add_rmsnorm(h, self.y, self.dest, self.topk_w, self.shared, self.gate, weight, out, eps, rows,
+                                    sum_weight=sum_weight, sum_eps=sum_eps)
+        return True
+
 
 register_part("feed_forward", "moe", MoeFeedForward)

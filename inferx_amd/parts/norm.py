@@ -44,26 +44,36 @@ class RMSNorm(Norm):
 
 class NormedDelta(LazyDelta):
     """A branch's result that passes a norm of its own before it is added to the residual stream (layers with a
-    norm before and after each branch): norm(tensor), not formed yet.  An RMS norm that consumes it forms it, adds
-    it and normalises the sum in one kernel; anybody else gets the normalised tensor in float32."""
+    norm before and after each branch): norm(delta), not formed yet.  `delta` may itself be a sum that is not formed
+    yet.  An RMS norm that consumes it forms it, adds it and normalises the sum in one kernel; anybody else gets the
+    normalised tensor in float32."""
 
-    def __init__(self, tensor, norm: Norm):
-        self.tensor, self.norm = tensor, norm
+    def __init__(self, delta, norm: Norm):
+        self.delta, self.norm = delta, norm
+
+    def tensor(self, ctx):
+        if isinstance(self.delta, LazyDelta):
+            self.delta = self.delta.materialize(ctx)
+        return self.delta
 
     def materialize(self, ctx):
-        zeros = torch.zeros(tuple(self.tensor.shape), dtype=torch.float32, device=self.tensor.device)
+        tensor = self.tensor(ctx)
+        zeros = torch.zeros(tuple(tensor.shape), dtype=torch.float32, device=tensor.device)
         rms = self.norm.rms_operands()
         if rms is None:  # some other norm: through its own forward, in the run's type
-            return self.norm.forward(ctx, zeros, self.tensor)
+            return self.norm.forward(ctx, zeros, tensor)
         out = torch.empty_like(zeros)
-        ops.add_rmsnorm(zeros, self.tensor, rms[0], out, rms[1])
+        ops.add_rmsnorm(zeros, tensor, rms[0], out, rms[1])
         return out
 
     def add_rmsnorm(self, ctx, h, weight, eps, rows, out) -> bool:
         rms = self.norm.rms_operands()
         if rms is None:
             return False
-        ops.add_normed_rmsnorm(h, self.tensor, rms[0], rms[1], weight, out, eps, rows)
+        fused = getattr(self.delta, "add_normed_rmsnorm", None)  # a sum that can be formed on the way
+        if fused is not None and fused(ctx, h, rms[0], rms[1], weight, eps, rows, out):
+            return True
+        ops.add_normed_rmsnorm(h, self.tensor(ctx), rms[0], rms[1], weight, out, eps, rows)
         return True
 
 

@@ -100,6 +100,37 @@ def test_normed_branch_add_and_norm(dtype, tol, width):
     close(hd, want_h, 2e-6, "the add alone")
 
 
+@pytest.mark.parametrize("dtype,tol", TYPES)
+@pytest.mark.parametrize("width,k", [(40, 1), (258, 3), (1000, 4)])
+def test_experts_sum_normed_added_and_normed(dtype, tol, width, k):
+    """The weighted sum of the chosen experts' rows, its own norm, the add and the next norm in one kernel."""
+    from inferx_amd import ops
+    T = 6
+    h = rnd((T, width), 1, 2.0)
+    y = rnd((T * k, width), 2, 1.0, dtype)
+    g = torch.Generator().manual_seed(3)
+    dest = torch.randperm(T * k, generator=g).to(torch.int32)
+    topk_w = torch.rand((T, k), generator=g)
+    wd, w = rnd((width,), 4) + 1.0, rnd((width,), 5) + 1.0
+    eps_d, eps = 1e-5, 1e-4
+    f = np.einsum("tk,tkw->tw", f64(topk_w), f64(y)[dest.long().numpy()].reshape(T, k, width))
+    want_h = f64(h) + pd.rms_norm(f, f64(wd), eps_d)
+    want = pd.rms_norm(want_h, f64(w), eps)
+    hd = h.to(DEV)
+    out = torch.empty((T, width), dtype=dtype, device=DEV)
+    ops.moe_combine_add_rmsnorm(hd, y.to(DEV), dest.to(DEV), topk_w.to(DEV), None, None, w.to(DEV), out, eps,
+                                sum_weight=wd.to(DEV), sum_eps=eps_d)
+    close(out, want, tol, "normalised rows")
+    close(hd, want_h, 2e-6, "the stream after the add")
+    hd = h.to(DEV)
+    rows = i32([4, 1])
+    out = torch.empty((2, width), dtype=dtype, device=DEV)
+    ops.moe_combine_add_rmsnorm(hd, y.to(DEV), dest.to(DEV), topk_w.to(DEV), None, None, w.to(DEV), out, eps, rows,
+                                sum_weight=wd.to(DEV), sum_eps=eps_d)
+    close(out, want[[4, 1]], tol, "picked rows")
+    assert torch.equal(hd.cpu(), h)
+
+
 # ---- the short convolution over steps, with silu, with rotation, into pages --------------------------------------
 @pytest.mark.parametrize("eights", [False, True])
 @pytest.mark.parametrize("taps", [1, 2, 4, 7])
