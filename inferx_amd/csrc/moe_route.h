@@ -82,7 +82,7 @@ template <int NW>
 __device__ __forceinline__ void
 select_dispatch_body(const float* logits, float* __restrict__ topk_w, int32_t* __restrict__ topk_e,
                      float* __restrict__ shared_gate, int32_t* __restrict__ offsets, int32_t* __restrict__ rows,
-                     int32_t* __restrict__ dest, int tokens, int experts, int k, int renormalize, float scale,
+                     int32_t* __restrict__ dest, int tokens, int experts, int k, int renormalize, float scale, int n_groups, int groups_keep,
                      int tile_rows, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
                      int32_t* __restrict__ tile_info) {
   static_assert(NW >= SD_MAX_EXPERTS / 64, "a thread per possible expert clears the counts");
@@ -115,6 +115,28 @@ select_dispatch_body(const float* logits, float* __restrict__ topk_w, int32_t* _
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
     const float inv_sum = 1.0f / sum;
+    if (groups_keep < n_groups) {
+      // equal groups of neighbouring experts (at most 64), scored by their best expert: the experts of all but the
+      // groups_keep best groups (among equals the lower number first) are struck out before the rounds below
+      const int per = experts / n_groups;
+      float best = -INFINITY;
+      if (lane < n_groups)
+        for (int e = lane * per; e < (lane + 1) * per; ++e) best = fmaxf(best, z[e]);
+      bool kept = false;
+      for (int round = 0; round < groups_keep; ++round) {
+        float bv = best;
+        int bi = lane < n_groups ? lane : 0x7fffffff;
+        ix_wave_argmax(bv, bi);
+        if (lane == bi) {
+          kept = true;
+          best = -INFINITY;
+        }
+      }
+      if (lane < n_groups && !kept)
+        for (int e = lane * per; e < (lane + 1) * per; ++e) z[e] = -INFINITY;
+      __builtin_amdgcn_wave_barrier();
+      __threadfence_block();
+    }
     float mine_w = 0.f, total = 0.f;
     for (int slot = 0; slot < k; ++slot) {
       float bv = -INFINITY;
@@ -228,7 +250,7 @@ template <int NW>
 __device__ __forceinline__ void
 select_dispatch_few(const float* logits, float* __restrict__ topk_w, int32_t* __restrict__ topk_e,
                     float* __restrict__ shared_gate, int32_t* __restrict__ offsets, int32_t* __restrict__ rows,
-                    int32_t* __restrict__ dest, int tokens, int experts, int k, int renormalize, float scale,
+                    int32_t* __restrict__ dest, int tokens, int experts, int k, int renormalize, float scale, int n_groups, int groups_keep,
                     int tile_rows, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
                     int32_t* __restrict__ tile_info) {
   auto fresh = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
@@ -260,6 +282,36 @@ select_dispatch_few(const float* logits, float* __restrict__ topk_w, int32_t* __
     }
     sum = ix_wave_sum(sum);
     const float inv_sum = 1.0f / sum;
+    if (groups_keep < n_groups) {  // (as in select_dispatch_body; lane g keeps the best score of group g)
+      const int per = experts / n_groups;
+      float best = -INFINITY;
+      for (int gi = 0; gi < n_groups; ++gi) {
+        float mg = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < SD_FEW_PER_LANE; ++j) {
+          const int e = lane + 64 * j;
+          if (e < experts && e / per == gi) mg = fmaxf(mg, z[j]);
+        }
+        mg = ix_wave_max(mg);
+        if (lane == gi) best = mg;
+      }
+      bool kept = false;
+      for (int round = 0; round < groups_keep; ++round) {
+        float bv = best;
+        int bi = lane < n_groups ? lane : 0x7fffffff;
+        ix_wave_argmax(bv, bi);
+        if (lane == bi) {
+          kept = true;
+          best = -INFINITY;
+        }
+      }
+      const unsigned long long kept_groups = __ballot(kept);
+#pragma unroll
+      for (int j = 0; j < SD_FEW_PER_LANE; ++j) {
+        const int e = lane + 64 * j;
+        if (e < experts && !((kept_groups >> (e / per)) & 1ull)) z[j] = -INFINITY;
+      }
+    }
     float mine_w = 0.f, total = 0.f;
     for (int slot = 0; slot < k; ++slot) {
       float bv = -INFINITY;

@@ -30,7 +30,7 @@ moe_route_dispatch_small_kernel(const T* __restrict__ x, float* h, const T* __re
                                 int32_t* arrived, int64_t width, float* __restrict__ topk_w,
                                 int32_t* __restrict__ topk_e, float* __restrict__ shared_gate,
                                 int32_t* __restrict__ offsets, int32_t* __restrict__ rows, int32_t* __restrict__ dest,
-                                int tokens, int experts, int k, int renormalize, float scale, int tile_rows,
+                                int tokens, int experts, int k, int renormalize, float scale, int n_groups, int groups_keep, int tile_rows,
                                 int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
                                 int32_t* __restrict__ tile_info) {
   extern __shared__ __align__(16) float xs[];  // [width]
@@ -109,10 +109,10 @@ moe_route_dispatch_small_kernel(const T* __restrict__ x, float* h, const T* __re
   if (tid == 0) __hip_atomic_store(arrived, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (tokens * k <= SD_FEW_ASSIGN)
     select_dispatch_few<RF_THREADS / 64>(logits, topk_w, topk_e, shared_gate, offsets, rows, dest, tokens, experts,
-                                         k, renormalize, scale, tile_rows, tile_expert, tile_row0, tile_info);
+                                         k, renormalize, scale, n_groups, groups_keep, tile_rows, tile_expert, tile_row0, tile_info);
   else
     select_dispatch_body<RF_THREADS / 64>(logits, topk_w, topk_e, shared_gate, offsets, rows, dest, tokens,
-                                          experts, k, renormalize, scale, tile_rows, tile_expert, tile_row0,
+                                          experts, k, renormalize, scale, n_groups, groups_keep, tile_rows, tile_expert, tile_row0,
                                           tile_info);
 }
 
@@ -121,12 +121,15 @@ static int route_dispatch_small_launch(const void* x, float* h, const void* delt
                                        const void* shared_gate_w, int sg_dtype, float* logits, int32_t* arrived,
                                        int64_t width, float* topk_w, int32_t* topk_e, float* shared_gate,
                                        int32_t* offsets, int32_t* rows, int32_t* dest, int tokens, int experts,
-                                       int k, int renormalize, float scale, int tile_rows, int32_t* tile_expert,
+                                       int k, int renormalize, float scale, int n_groups, int groups_keep, int tile_rows, int32_t* tile_expert,
                                        int32_t* tile_row0, int32_t* tile_info, hipStream_t stream) {
   IX_REQUIRE(tokens > 0 && tokens <= 16 && experts > 0 && k > 0 && width > 0, "between 1 and 16 tokens, sizes positive");
   IX_REQUIRE(dtype == IX_F32 || dtype == IX_BF16, "dtype must be float32 or bfloat16");
   IX_REQUIRE(experts <= SD_MAX_EXPERTS, "at most 256 experts for the one-workgroup selection");
   IX_REQUIRE(k <= experts && k <= 32, "top_k must be between 1 and min(experts, 32)");
+  IX_REQUIRE(n_groups >= 1 && n_groups <= 64 && experts % n_groups == 0 && groups_keep >= 1 && groups_keep <= n_groups &&
+                 k <= groups_keep * (experts / n_groups),
+             "between 1 and 64 equal groups of experts, of which the kept ones must hold top_k experts");
   IX_REQUIRE(static_cast<int64_t>(tokens) * k <= SD_MAX_ASSIGN, "at most 1024 assignments for the one-workgroup selection");
   IX_REQUIRE(tile_rows >= 0, "tile_rows must not be negative");
   IX_REQUIRE(tile_rows == 0 || (tile_expert && tile_row0 && tile_info), "tile map buffers needed");
@@ -139,7 +142,7 @@ static int route_dispatch_small_launch(const void* x, float* h, const void* delt
   hipLaunchKernelGGL((moe_route_dispatch_small_kernel<T, NORM>), grid, block, xs_bytes, stream, (const T*)x, h,     \
                      (const T*)delta, gamma, gamma_dtype, eps, (T*)x_out, wr, wr_dtype, shared_gate_w, sg_dtype,    \
                      logits, arrived, width, topk_w, topk_e, shared_gate, offsets, rows, dest, tokens, experts, k,  \
-                     renormalize, scale, tile_rows, tile_expert, tile_row0, tile_info)
+                     renormalize, scale, n_groups, groups_keep, tile_rows, tile_expert, tile_row0, tile_info)
   if (h) {
     if (dtype == IX_F32) LAUNCH(float, true);
     else LAUNCH(bf16_t, true);
@@ -158,12 +161,12 @@ extern "C" int ix_moe_route_dispatch_small(const void* x, int dtype, const void*
                                            const void* shared_gate_w, int sg_dtype, float* logits, int32_t* arrived,
                                            int64_t width, float* topk_w, int32_t* topk_e, float* shared_gate,
                                            int32_t* offsets, int32_t* rows, int32_t* dest, int tokens, int experts,
-                                           int k, int renormalize, float scale, int tile_rows, int32_t* tile_expert,
+                                           int k, int renormalize, float scale, int n_groups, int groups_keep, int tile_rows, int32_t* tile_expert,
                                            int32_t* tile_row0, int32_t* tile_info, hipStream_t stream) {
   IX_REQUIRE(x != nullptr, "x needed");
   return route_dispatch_small_launch(x, nullptr, nullptr, nullptr, IX_F32, 0.f, nullptr, dtype, wr, wr_dtype,
                                      shared_gate_w, sg_dtype, logits, arrived, width, topk_w, topk_e, shared_gate,
-                                     offsets, rows, dest, tokens, experts, k, renormalize, scale, tile_rows,
+                                     offsets, rows, dest, tokens, experts, k, renormalize, scale, n_groups, groups_keep, tile_rows,
                                      tile_expert, tile_row0, tile_info, stream);
 }
 
@@ -174,13 +177,13 @@ extern "C" int ix_moe_norm_route_dispatch_small(float* h, const void* delta, int
                                                 const void* shared_gate_w, int sg_dtype, float* logits,
                                                 int32_t* arrived, int64_t width, float* topk_w, int32_t* topk_e,
                                                 float* shared_gate, int32_t* offsets, int32_t* rows, int32_t* dest,
-                                                int tokens, int experts, int k, int renormalize, float scale,
+                                                int tokens, int experts, int k, int renormalize, float scale, int n_groups, int groups_keep,
                                                 int tile_rows, int32_t* tile_expert, int32_t* tile_row0,
                                                 int32_t* tile_info, hipStream_t stream) {
   IX_REQUIRE(h && delta && gamma && x_out, "h, delta, gamma and x_out needed");
   IX_REQUIRE(gamma_dtype == IX_F32 || gamma_dtype == IX_BF16, "the norm weight must be float32 or bfloat16");
   return route_dispatch_small_launch(nullptr, h, delta, gamma, gamma_dtype, eps, x_out, dtype, wr, wr_dtype,
                                      shared_gate_w, sg_dtype, logits, arrived, width, topk_w, topk_e, shared_gate,
-                                     offsets, rows, dest, tokens, experts, k, renormalize, scale, tile_rows,
+                                     offsets, rows, dest, tokens, experts, k, renormalize, scale, n_groups, groups_keep, tile_rows,
                                      tile_expert, tile_row0, tile_info, stream);
 }

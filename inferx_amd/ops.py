@@ -375,7 +375,7 @@ def moe_route_dispatch(x: Optional[torch.Tensor], router_w: torch.Tensor, shared
                        topk_w: torch.Tensor, topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor],
                        renormalize: bool, scale: float, offsets: torch.Tensor, rows: torch.Tensor,
                        dest: torch.Tensor, tile_rows: int = 0, tile_map: Optional[torch.Tensor] = None,
-                       norm: Optional[tuple] = None) -> None:
+                       norm: Optional[tuple] = None, groups: int = 1, groups_keep: int = 1) -> None:
     """`moe_route` and `moe_dispatch` for up to 16 tokens in one launch: the router scores are spread over many
     workgroups, and the last one to finish its scores selects and groups (`route_one_launch_fits`).
 
@@ -394,6 +394,8 @@ def moe_route_dispatch(x: Optional[torch.Tensor], router_w: torch.Tensor, shared
     k = topk_w.shape[1]
     A = T * k
     _need(route_one_launch_fits(T, H, E), "too many tokens or experts, or too wide, for the one-launch router")
+    _need(1 <= groups <= 64 and E % groups == 0 and 1 <= groups_keep <= groups and k <= groups_keep * (E // groups),
+          "the experts must split into at most 64 equal groups, and the kept groups must hold top_k experts")
     _need(router_w.shape == (E, H), "router weight must be [experts, hidden]")
     _need(topk_w.shape == (T, k) and topk_w.dtype == torch.float32, "topk_w must be float32 [T, k]")
     _need(topk_e.shape == (T, k) and topk_e.dtype == torch.int32, "topk_e must be int32 [T, k]")
@@ -415,8 +417,8 @@ def moe_route_dispatch(x: Optional[torch.Tensor], router_w: torch.Tensor, shared
               _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(logits),
               _ptr(_arrival_counter(x.device)), _i64(H), _ptr(topk_w), _ptr(topk_e),
               _ptr(shared_gate if shared_gate_w is not None else None), _ptr(offsets), _ptr(rows), _ptr(dest),
-              _i32(T), _i32(E), _i32(k), _i32(1 if renormalize else 0), _f32(scale), _i32(tile_rows), _ptr(te),
-              _ptr(tr), _ptr(ti), _stream())
+              _i32(T), _i32(E), _i32(k), _i32(1 if renormalize else 0), _f32(scale), _i32(groups), _i32(groups_keep),
+              _i32(tile_rows), _ptr(te), _ptr(tr), _ptr(ti), _stream())
     if norm is not None:
         _call("ix_moe_norm_route_dispatch_small", _ptr(h), _ptr(delta), _i32(_dt(x_out)), _ptr(gamma),
               _i32(_dt(gamma)), _f32(eps), _ptr(x_out), *router)

@@ -219,14 +219,13 @@ class MoeFeedForward(FeedForward):
         dest = rt.empty((T * k,), torch.int32)
         tile_map = rt.empty((2 * ops.moe_max_tiles(T * k, E, tile_rows) + 1,), torch.int32) if tile_rows else None
         ops.moe_route_dispatch(None if norm else x, self.w_router, self.w_shared_gate, topk_w, topk_e, gate,
-                               self.renormalize, self.routed_scale, offsets, rows, dest, tile_rows, tile_map, norm)
+                               self.renormalize, self.routed_scale, offsets, rows, dest, tile_rows, tile_map, norm,
+                               self.groups, self.groups_keep)
         return topk_w, topk_e, gate, offsets, rows, dest, tile_map
 
     def _routes_in_one_launch(self, tokens: int) -> bool:
-        """Whether the router's scores, selection and grouping of this step fit the one launch for few tokens (which
-        chooses among all experts: a router that keeps only some groups goes through the separate kernels)."""
-        return self.groups_keep == self.groups and ops.route_one_launch_fits(tokens, self.hidden_size,
-                                                                             self.num_experts)
+        """Whether the router's scores, selection and grouping of this step fit the one launch for few tokens."""
+        return ops.route_one_launch_fits(tokens, self.hidden_size, self.num_experts)
 
     takes_lazy_norm = True
 

@@ -18,7 +18,7 @@ import tiny_dezudra as td
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LENGTHS = {"A": (5, 9, 27, 70), "B": (7, 23, 40, 75), "C": (1, 2, 33, 70), "D": (3, 50, 66)}
+LENGTHS = {"A": (5, 9, 27, 70), "B": (7, 23, 40, 75), "C": (1, 2, 33, 70), "D": (3, 50, 66), "E": (4, 19, 45), "F": (6, 31, 52)}
 # relative to the largest |logit| of the expected rows; fixed before the first run
 TOL = {"float32": ru.FP32_TOL, "bfloat16": ru.BF16_TOL}
 NAMES = sorted(td.CONFIGS)
@@ -184,8 +184,10 @@ def test_mixed_batches_with_few_pages(folders, name, dtype, monkeypatch):
     run_and_check(folders, name, dtype, steps, monkeypatch, f"mixed {name} {dtype}", prompts, num_pages=max_tokens // 16)
     # the same steps once more, to see that pages really are used again
     owners = {}
-    ru.replay(make_runner(folders, name, dtype, num_pages=max_tokens // 16), steps, page_owners=owners)
-    assert any(len(who) > 1 for who in owners.values()), "no physical page was used by two requests"
+    runner = make_runner(folders, name, dtype, num_pages=max_tokens // 16)
+    ru.replay(runner, steps, page_owners=owners)
+    if runner.cache.groups:  # (a model of recurrent layers only keeps nothing in pages)
+        assert any(len(who) > 1 for who in owners.values()), "no physical page was used by two requests"
 
 
 @pytest.mark.parametrize("name", ["A", "B"])

@@ -372,13 +372,13 @@ def test_one_key_stands_out_at_every_edge(dtype):
     the kept first tokens and the ones after them, page borders, far keys; for queries at many positions."""
     from inferx_amd import ops
     H, G, D, V, L, page = 2, 1, 16, 24, 1100, 16
-    window, keep = 40, 5
+    window, keep = 37, 5
     k = rnd((L, 2 * G, D), 1, 0.05)
     v = rnd((L, G, V), 2, 1.0)
     mark = torch.zeros(D)
     mark[7] = 1.0
     lam, eps, mult = 0.0, 1e-6, 1.0  # lambda 0: the result is map 0's alone
-    for pos in (39, 40, 41, 47, 48, 300, 1023, 1024, 1099):
+    for pos in (36, 37, 38, 47, 48, 300, 1023, 1024, 1099):
         cases = {0: True, keep - 1: True, keep: pos - keep < window, 15: pos - 15 < window, 16: pos - 16 < window,
                  pos - window + 1: True, pos - window: pos - window < keep, pos - window - 1: pos - window - 1 < keep,
                  pos: True, (pos // page) * page: True, (pos // page) * page - 1: pos - ((pos // page) * page - 1) < window}
@@ -401,12 +401,14 @@ def test_one_key_stands_out_at_every_edge(dtype):
 
 # ---- experts of squared relu, chosen among groups ---------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,tol", TYPES)
-@pytest.mark.parametrize("tokens", [3, 40, 300])
+@pytest.mark.parametrize("tokens", [3, 16, 40, 300])
 @pytest.mark.parametrize("E,top,groups,keep,ff,width", [(6, 2, 3, 2, 64, 96), (9, 3, 3, 1, 52, 72), (16, 4, 8, 3, 32, 128),
-                                                        (4, 4, 2, 2, 40, 40), (5, 1, 1, 1, 36, 72), (2, 1, 2, 1, 24, 40)])
+                                                        (4, 4, 2, 2, 40, 40), (5, 1, 1, 1, 36, 72), (2, 1, 2, 1, 24, 40),
+                                                        (16, 6, 4, 2, 32, 128), (128, 5, 16, 3, 16, 64)])
 def test_experts_chosen_among_groups(dtype, tol, tokens, E, top, groups, keep, ff, width):
     """The feed-forward part as the design builds it, against the plain one: choices (where no near tie), weights and
-    the weighted sum; few tokens (the streaming kernels), some (16-row tiles) and many (tiles through LDS)."""
+    the weighted sum; few tokens (the streaming kernels, and the router, selection and grouping in one launch: up to 64
+    assignments in registers, more through LDS), some (16-row tiles) and many (tiles through LDS)."""
     from inferx_amd.engine.runtime import Runtime, StepContext
     from inferx_amd.parts.base import resolve_delta
     from inferx_amd.parts.moe import MoeFeedForward
@@ -428,7 +430,7 @@ def test_experts_chosen_among_groups(dtype, tol, tokens, E, top, groups, keep, f
     margins = []
     s, ids, wts = pd.route(f64(x), mlp["router"], Wn["router"], margins)
     sure = margins[0] > (1e-6 if dtype == torch.float32 else 3e-2)
-    assert sure.sum() >= tokens // 2
+    assert sure.sum() >= tokens // 3
     assert np.array_equal(topk_e.cpu().numpy()[sure], ids[sure]), "another choice of experts"
     close(topk_w.cpu()[torch.from_numpy(sure)], wts[sure], tol, "weights")
     got = resolve_delta(ctx, part.forward(ctx, x.to(DEV)))
@@ -481,7 +483,7 @@ def test_differential_attention_on_the_matrix_cores(H, G, D, V, window, keep, n_
 
 
 @pytest.mark.parametrize("n_splits", [1, 4])
-@pytest.mark.parametrize("H,G,D,V,window,keep", [(4, 2, 32, 32, 24, 3), (16, 1, 64, 32, 0, 0), (6, 2, 16, 96, 40, 4)])
+@pytest.mark.parametrize("H,G,D,V,window,keep", [(4, 2, 32, 32, 24, 3), (16, 1, 64, 32, 0, 0), (6, 2, 16, 96, 44, 3)])
 def test_differential_attention_one_token_each_grouped(H, G, D, V, window, keep, n_splits):
     """Three requests of unequal contexts, one token each, the query heads of a key/value head side by side."""
     dtype = torch.bfloat16
@@ -517,14 +519,14 @@ def test_one_key_stands_out_at_every_edge_on_the_matrix_cores(grouped):
     """As the plain kernel's test: one key far above the others is found exactly where the window and the kept
     first tokens say, also when the pages between them hold not-a-number (they may have been given back)."""
     H, G, D, V, L, page = 2, 1, 16, 32, 1100, 16
-    window, keep = 40, 5
+    window, keep = 37, 5
     dtype = torch.bfloat16
     k = rnd((L, 2 * G, D), 1, 0.05)
     v = rnd((L, G, V), 2, 1.0)
     mark = torch.zeros(D)
     mark[7] = 1.0
     lam, eps, mult = 0.0, 1e-6, 1.0
-    for pos in (39, 40, 41, 47, 48, 300, 1023, 1024, 1099):
+    for pos in (36, 37, 38, 47, 48, 300, 1023, 1024, 1099):
         cases = {0: True, keep - 1: True, keep: pos - keep < window, 15: pos - 15 < window, 16: pos - 16 < window,
                  pos - window + 1: True, pos - window: pos - window < keep, pos - window - 1: pos - window - 1 < keep,
                  pos: True, (pos // page) * page: True, (pos // page) * page - 1: pos - ((pos // page) * page - 1) < window}

@@ -35,7 +35,7 @@ def config(vocab, width, eps, logit_scale, layers):
 # A: attention first, then the recurrent mixer; matrix-core sizes; three groups of which two are kept; windows of
 # two sizes, one that keeps no first tokens
 A = config(320, 96, 1e-5, 0.5, [
-    attention(4, 2, 32, 32, 4, 0.2, 0.3, (32, 10000.0), (24, 3), experts(64, 6, 2, (3, 2))),
+    attention(6, 2, 32, 32, 4, 0.2, 0.3, (32, 10000.0), (24, 3), experts(64, 6, 2, (3, 2))),
     delta(4, 4, 16, 48, 2, experts(64, 6, 2, (3, 2))),
     attention(2, 2, 16, 48, 2, 0.3, 0.8, (8, 500.0), (9, 0), experts(40, 4, 4, (2, 2))),
 ])
@@ -58,7 +58,22 @@ D = config(256, 128, 1e-5, 0.25, [
     delta(2, 1, 128, 80, 4, experts(32, 16, 4, (4, 2))),
     attention(4, 1, 64, 96, 4, 0.125, 0.4, (32, 1000.0), (33, 1), experts(32, 16, 4, (8, 3))),
 ])
-CONFIGS = {"A": A, "B": B, "C": C, "D": D}
+# E: recurrent layers only (nothing is kept in pages), a width and a vocabulary that are no multiple of 8, groups of one
+# expert, the logits' scale left to its default
+E = config(77, 90, 1e-5, 1.0, [
+    delta(2, 1, 24, 20, 3, experts(28, 6, 2, (6, 3))),
+    delta(3, 3, 10, 14, 2, experts(28, 3, 1, (1, 1))),
+])
+del E["logit_scale"]
+# F: attention layers only, key/value heads omitted (as many as heads), values as wide as keys by omission, more
+# query heads per key/value head than a tile has columns
+F = config(203, 104, 1e-6, 0.125, [
+    attention(5, 5, 16, 16, 2, 0.3, 0.25, (6, 77.0), (11, 1), experts(44, 8, 3, (4, 2))),
+    attention(34, 1, 16, 8, 3, 0.2, 0.7, None, (5, 6), experts(44, 8, 8, (2, 2))),
+])
+for _name in ("kv_heads", "vdim"):
+    del F["layers"][0]["mixer"][_name]
+CONFIGS = {"A": A, "B": B, "C": C, "D": D, "E": E, "F": F}
 
 
 def make_folder(raw_config: dict, seed: int, out_dir: str, dtype: str = "bfloat16") -> str:
