@@ -226,30 +226,41 @@ attn_diff_combine_kernel(const float* __restrict__ part_o, const float* __restri
   const int64_t th = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);  // token * heads + head
   if (th >= pairs) return;
   const int lane = threadIdx.x & 63;
-  float a[2][4];
+  // both maps' reference points and sums are asked for first, then all parts: the loads of a launch this small
+  // should all be in flight together
+  float a[2][4], w[2], inv_l[2];
+  float m_s[2], l_s[2];
 #pragma unroll
   for (int mp = 0; mp < 2; ++mp) {
     const int64_t p0 = (th * 2 + mp) * n_splits;
-    const float m_s = lane < n_splits ? part_ml[2 * (p0 + lane)] : -INFINITY;
-    const float l_s = lane < n_splits ? part_ml[2 * (p0 + lane) + 1] : 0.f;
-    const float M = ix_wave_max(m_s);
-    const float w = (m_s == -INFINITY) ? 0.f : exp2f(m_s - M);
-    const float inv_l = 1.0f / ix_wave_sum(w * l_s);
+    m_s[mp] = lane < n_splits ? part_ml[2 * (p0 + lane)] : -INFINITY;
+    l_s[mp] = lane < n_splits ? part_ml[2 * (p0 + lane) + 1] : 0.f;
+  }
+#pragma unroll
+  for (int mp = 0; mp < 2; ++mp) {
+    const float M = ix_wave_max(m_s[mp]);
+    w[mp] = (m_s[mp] == -INFINITY) ? 0.f : exp2f(m_s[mp] - M);
+    inv_l[mp] = 1.0f / ix_wave_sum(w[mp] * l_s[mp]);
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) a[mp][jj] = 0.f;
-    // (columns past the head's end read its last column again: every load is unconditional, so that the loads of
-    // several slices are in flight together; what they sum is dropped below)
-#pragma unroll 4
-    for (int s = 0; s < n_splits; ++s) {
-      const float ws = __shfl(w, s, 64);
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        if (64 * jj < value_dim) a[mp][jj] += ws * part_o[(p0 + s) * value_dim + min(lane + 64 * jj, value_dim - 1)];
-      }
-    }
-#pragma unroll
-    for (int jj = 0; jj < 4; ++jj) a[mp][jj] *= inv_l;
   }
+  // (columns past the head's end read its last column again: every load is unconditional; what they sum is dropped)
+  const float* po = part_o + th * 2 * n_splits * value_dim;
+#pragma unroll 4
+  for (int s = 0; s < n_splits; ++s) {
+#pragma unroll
+    for (int mp = 0; mp < 2; ++mp) {
+      const float ws = __shfl(w[mp], s, 64);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj)
+        if (64 * jj < value_dim)
+          a[mp][jj] += ws * po[static_cast<int64_t>(mp * n_splits + s) * value_dim + min(lane + 64 * jj, value_dim - 1)];
+    }
+  }
+#pragma unroll
+  for (int mp = 0; mp < 2; ++mp)
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) a[mp][jj] *= inv_l[mp];
   float ss = 0.f;
 #pragma unroll
   for (int jj = 0; jj < 4; ++jj) {

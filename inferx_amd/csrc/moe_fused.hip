@@ -79,7 +79,8 @@ __global__ void moe_combine_add_rmsnorm_vec4_kernel(float* __restrict__ h, const
                                                     const uint16_t* __restrict__ shared,
                                                     const float* __restrict__ shared_gate, const void* __restrict__ w,
                                                     int w_dtype, uint16_t* __restrict__ out,
-                                                    const int32_t* __restrict__ rows, int64_t width, int k, float eps) {
+                                                    const int32_t* __restrict__ rows, int64_t width, int k, float eps,
+                                                    const void* __restrict__ wd, int wd_dtype, float eps_d) {
   extern __shared__ __align__(16) float vrow[];  // [width]
   __shared__ float red[16];
   __shared__ float sw[32];
@@ -94,6 +95,27 @@ __global__ void moe_combine_add_rmsnorm_vec4_kernel(float* __restrict__ h, const
   const float sg = shared ? (shared_gate ? shared_gate[row] : 1.0f) : 0.f;
   float* hr = h + row * width;
   float sumsq = 0.f;
+  float inv_d = 1.0f;
+  if (wd) {  // the sum is normalised before it is added: its sum of squares first (the sum itself is formed twice)
+    float sumsq_d = 0.f;
+    for (int64_t c = 4 * threadIdx.x; c < width; c += 4 * blockDim.x) {
+      float acc[4] = {0.f, 0.f, 0.f, 0.f}, f[4];
+      for (int s = 0; s < k; ++s) {
+        bf16x4_to_f32(*reinterpret_cast<const uint2*>(y + static_cast<int64_t>(sd[s]) * width + c), f);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += sw[s] * f[i];
+      }
+      if (shared) {
+        bf16x4_to_f32(*reinterpret_cast<const uint2*>(shared + row * width + c), f);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += sg * f[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sumsq_d += acc[i] * acc[i];
+    }
+    sumsq_d = ix_block_sum(sumsq_d, red);
+    inv_d = 1.0f / sqrtf(sumsq_d / static_cast<float>(width) + eps_d);
+  }
   for (int64_t c = 4 * threadIdx.x; c < width; c += 4 * blockDim.x) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f}, f[4];
     for (int s = 0; s < k; ++s) {
@@ -105,6 +127,10 @@ __global__ void moe_combine_add_rmsnorm_vec4_kernel(float* __restrict__ h, const
       bf16x4_to_f32(*reinterpret_cast<const uint2*>(shared + row * width + c), f);
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[i] += sg * f[i];
+    }
+    if (wd) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] *= inv_d * ix_load_rt(wd, wd_dtype, c + i);
     }
     float4 v = *reinterpret_cast<const float4*>(hr + c);
     v.x += acc[0]; v.y += acc[1]; v.z += acc[2]; v.w += acc[3];
@@ -145,12 +171,12 @@ extern "C" int ix_moe_combine_add_rmsnorm(void* h, const void* y, int dtype, con
     hipLaunchKernelGGL(moe_combine_add_rmsnorm_kernel<float>, grid, block, smem, stream, (float*)h, (const float*)y,
                        dest, topk_w, (const float*)shared, shared_gate, w, w_dtype, (float*)out, rows, width, k, eps, wd,
                        wd_dtype, eps_d);
-  else if (dtype == IX_BF16 && wd == nullptr && width % 4 == 0 &&
+  else if (dtype == IX_BF16 && width % 4 == 0 &&
            ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(shared) |
              reinterpret_cast<uintptr_t>(out)) & 15) == 0)
     hipLaunchKernelGGL(moe_combine_add_rmsnorm_vec4_kernel, grid, dim3(width >= 4096 ? 1024 : (width >= 2048 ? 512 : 256)),
                        smem, stream, (float*)h, (const uint16_t*)y, dest, topk_w, (const uint16_t*)shared, shared_gate, w,
-                       w_dtype, (uint16_t*)out, rows, width, k, eps);
+                       w_dtype, (uint16_t*)out, rows, width, k, eps, wd, wd_dtype, eps_d);
   else if (dtype == IX_BF16)
     hipLaunchKernelGGL(moe_combine_add_rmsnorm_kernel<bf16_t>, grid, block, smem, stream, (float*)h,
                        (const bf16_t*)y, dest, topk_w, (const bf16_t*)shared, shared_gate, w, w_dtype, (bf16_t*)out,

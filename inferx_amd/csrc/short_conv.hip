@@ -209,14 +209,39 @@ __device__ __forceinline__ Conv8 conv_at8(const ConvArgs& a, const float* wt, co
   Conv8 y;
 #pragma unroll
   for (int e = 0; e < 8; ++e) y.x[e] = 0.f;
-  for (int j = 0; j < a.taps; ++j) {
-    const Conv8 u = conv_input8(a, bias_f, in, st, row0, i - a.taps + 1 + j, c);
-    const float* wr = wt + static_cast<int64_t>(j) * a.channels + c;
-    const conv_f32x4 w0 = *reinterpret_cast<const conv_f32x4*>(wr), w1 = *reinterpret_cast<const conv_f32x4*>(wr + 4);
+  if (a.taps <= 4) {
+    // up to four taps: every input and every tap is asked for before the first is used (one trip to memory
+    // instead of one per tap, which is what a step of few tokens waits for); the same sums in the same order
+    Conv8 u[4];
+    conv_f32x4 w0[4], w1[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      y.x[e] += w0[e] * u.x[e];
-      y.x[4 + e] += w1[e] * u.x[4 + e];
+    for (int j = 0; j < 4; ++j) {
+      const int jj = min(j, a.taps - 1);
+      u[j] = conv_input8(a, bias_f, in, st, row0, i - a.taps + 1 + jj, c);
+      const float* wr = wt + static_cast<int64_t>(jj) * a.channels + c;
+      w0[j] = *reinterpret_cast<const conv_f32x4*>(wr);
+      w1[j] = *reinterpret_cast<const conv_f32x4*>(wr + 4);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (j < a.taps) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          y.x[e] += w0[j][e] * u[j].x[e];
+          y.x[4 + e] += w1[j][e] * u[j].x[4 + e];
+        }
+      }
+    }
+  } else {
+    for (int j = 0; j < a.taps; ++j) {
+      const Conv8 u = conv_input8(a, bias_f, in, st, row0, i - a.taps + 1 + j, c);
+      const float* wr = wt + static_cast<int64_t>(j) * a.channels + c;
+      const conv_f32x4 w0 = *reinterpret_cast<const conv_f32x4*>(wr), w1 = *reinterpret_cast<const conv_f32x4*>(wr + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        y.x[e] += w0[e] * u.x[e];
+        y.x[4 + e] += w1[e] * u.x[4 + e];
+      }
     }
   }
   if (a.silu) {
