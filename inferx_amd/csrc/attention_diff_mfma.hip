@@ -219,10 +219,14 @@ attn_diff_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k
 
 // Per (token, head), one wavefront: both maps' slices merged (a_m = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M)),
 // o = a_0 - lambda a_1, out = o / sqrt(mean(o^2) + eps) * mult.  At most 64 slices, value_dim at most 256.
+// NS: the number of slices where it is 1, 2, 4 or 8 (the loop over them is then unrolled whole, so that every load of
+// the launch is in flight at once), else 0.
+template <int NS>
 __global__ void __launch_bounds__(256)
 attn_diff_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                         __bf16* __restrict__ out, int64_t pairs, int n_splits, int value_dim, float lambda, float eps,
-                         float mult) {
+                         __bf16* __restrict__ out, int64_t pairs, int n_splits_any, int value_dim, float lambda,
+                         float eps, float mult) {
+  const int n_splits = NS > 0 ? NS : n_splits_any;
   const int64_t th = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);  // token * heads + head
   if (th >= pairs) return;
   const int lane = threadIdx.x & 63;
@@ -230,6 +234,20 @@ attn_diff_combine_kernel(const float* __restrict__ part_o, const float* __restri
   // should all be in flight together
   float a[2][4], w[2], inv_l[2];
   float m_s[2], l_s[2];
+  const float* po = part_o + th * 2 * n_splits * value_dim;
+  // (columns past the head's end read its last column again: every load is unconditional; what they sum is dropped)
+  float parts[2][NS > 0 ? NS : 1][4];
+  if constexpr (NS > 0) {  // the parts themselves first: they wait for nothing
+#pragma unroll
+    for (int mp = 0; mp < 2; ++mp)
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+          parts[mp][s][jj] = 64 * jj < value_dim
+                                 ? po[static_cast<int64_t>(mp * NS + s) * value_dim + min(lane + 64 * jj, value_dim - 1)]
+                                 : 0.f;
+  }
 #pragma unroll
   for (int mp = 0; mp < 2; ++mp) {
     const int64_t p0 = (th * 2 + mp) * n_splits;
@@ -244,10 +262,7 @@ attn_diff_combine_kernel(const float* __restrict__ part_o, const float* __restri
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) a[mp][jj] = 0.f;
   }
-  // (columns past the head's end read its last column again: every load is unconditional; what they sum is dropped)
-  const float* po = part_o + th * 2 * n_splits * value_dim;
-#pragma unroll 4
-  for (int s = 0; s < n_splits; ++s) {
+  auto take = [&](int s) {
 #pragma unroll
     for (int mp = 0; mp < 2; ++mp) {
       const float ws = __shfl(w[mp], s, 64);
@@ -256,6 +271,19 @@ attn_diff_combine_kernel(const float* __restrict__ part_o, const float* __restri
         if (64 * jj < value_dim)
           a[mp][jj] += ws * po[static_cast<int64_t>(mp * n_splits + s) * value_dim + min(lane + 64 * jj, value_dim - 1)];
     }
+  };
+  if constexpr (NS > 0) {
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+      for (int mp = 0; mp < 2; ++mp) {
+        const float ws = __shfl(w[mp], s, 64);
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) a[mp][jj] += ws * parts[mp][s][jj];
+      }
+  } else {
+#pragma unroll 4
+    for (int s = 0; s < n_splits; ++s) take(s);
   }
 #pragma unroll
   for (int mp = 0; mp < 2; ++mp)
@@ -349,7 +377,16 @@ extern "C" int ix_attention_diff_mfma(const void* q, const void* k_cache, const 
 #undef ARGS
   if (ix_check_launch("ix_attention_diff_mfma")) return 1;
   const int64_t pairs = tokens * heads;
-  hipLaunchKernelGGL(attn_diff_combine_kernel, dim3(static_cast<unsigned>((pairs + 3) / 4)), dim3(256), 0, stream, part_o,
-                     part_ml, (__bf16*)out, pairs, n_splits, value_dim, lambda, eps, mult);
+#define MERGE(NS)                                                                                                   \
+  hipLaunchKernelGGL(attn_diff_combine_kernel<NS>, dim3(static_cast<unsigned>((pairs + 3) / 4)), dim3(256), 0, stream, \
+                     part_o, part_ml, (__bf16*)out, pairs, n_splits, value_dim, lambda, eps, mult)
+  switch (n_splits) {
+    case 1: MERGE(1); break;
+    case 2: MERGE(2); break;
+    case 4: MERGE(4); break;
+    case 8: MERGE(8); break;
+    default: MERGE(0); break;
+  }
+#undef MERGE
   return ix_check_launch("ix_attention_diff_mfma (merge)");
 }
