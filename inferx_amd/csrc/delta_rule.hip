@@ -15,6 +15,9 @@
 // start and written back at the end.  Query head h reads the q/k head h / (heads / kv_heads).
 #include "common.h"
 
+typedef unsigned int delta_u32x4 __attribute__((ext_vector_type(4)));
+typedef float delta_f32x4 __attribute__((ext_vector_type(4)));
+
 #define DELTA_COLS 16   // value columns per wavefront
 #define DELTA_SPLIT 4   // lanes per column
 
@@ -53,11 +56,26 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
   // the rows of this lane: VEC part * dim / 4 + r, else r * 4 + part
   const int quarter = dim / DELTA_SPLIT;
   auto row_of = [&](int r) { return VEC ? (r < quarter ? part * quarter + r : dim) : r * DELTA_SPLIT + part; };
+  // the state keeps a column's rows side by side ([head][column][row]): a lane's rows are one run of memory
   float S[RPL];
+  if constexpr (VEC) {  // (the entry point has seen to it that the runs are 16-byte aligned)
 #pragma unroll
-  for (int r = 0; r < RPL; ++r) {
-    const int i = row_of(r);
-    S[r] = i < dim ? sp[static_cast<int64_t>(i) * vdim + cj] : 0.f;
+    for (int r = 0; r < RPL; r += 4) {
+      if (r < quarter) {
+        const delta_f32x4 x = *reinterpret_cast<const delta_f32x4*>(sp + static_cast<int64_t>(cj) * dim + part * quarter + r);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) S[r + e] = x[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) S[r + e] = 0.f;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) {
+      const int i = row_of(r);
+      S[r] = i < dim ? sp[static_cast<int64_t>(cj) * dim + i] : 0.f;
+    }
   }
   const float rate = expf(a_log[head]), bias = dt_bias[head];
   const float q_scale = 1.0f / sqrtf(static_cast<float>(dim));
@@ -142,10 +160,18 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
     bc = bn;
   }
   if (live) {
+    if constexpr (VEC) {
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) {
-      const int i = row_of(r);
-      if (i < dim) sp[static_cast<int64_t>(i) * vdim + col] = S[r];
+      for (int r = 0; r < RPL; r += 4)
+        if (r < quarter)
+          *reinterpret_cast<delta_f32x4*>(sp + static_cast<int64_t>(col) * dim + part * quarter + r) =
+              delta_f32x4{S[r], S[r + 1], S[r + 2], S[r + 3]};
+    } else {
+#pragma unroll
+      for (int r = 0; r < RPL; ++r) {
+        const int i = row_of(r);
+        if (i < dim) sp[static_cast<int64_t>(col) * dim + i] = S[r];
+      }
     }
   }
 }
@@ -163,8 +189,6 @@ delta_rule_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __r
 // Per row and lane that leaves four sweeps over RPL numbers and two sums over SP lanes.  (The decay is applied to
 // the product S^T k instead of to S first, which is the same number up to rounding.)
 #define DELTA_CHUNK 32
-typedef unsigned int delta_u32x4 __attribute__((ext_vector_type(4)));
-typedef float delta_f32x4 __attribute__((ext_vector_type(4)));
 
 template <int SP>
 __device__ __forceinline__ float delta_sum_over(float x) {  // over the SP neighbouring lanes of a column
@@ -204,7 +228,7 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
   float* sp = state + static_cast<int64_t>(state_slots[seq]) * state_stride + static_cast<int64_t>(head) * DIM * vdim;
   float S[RPL];
 #pragma unroll
-  for (int r = 0; r < RPL; ++r) S[r] = sp[static_cast<int64_t>(part * RPL + r) * vdim + cj];
+  for (int r = 0; r < RPL; ++r) S[r] = sp[static_cast<int64_t>(cj) * DIM + part * RPL + r];
   const float rate = expf(a_log[head]), bias = dt_bias[head];
   const float q_scale = 1.0f / sqrtf(static_cast<float>(DIM));
 
@@ -314,12 +338,12 @@ delta_rule_chunk_kernel(const bf16_t* q, const bf16_t* k, const bf16_t* v, int64
   }
   if (live) {
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) sp[static_cast<int64_t>(part * RPL + r) * vdim + col] = S[r];
+    for (int r = 0; r < RPL; ++r) sp[static_cast<int64_t>(col) * DIM + part * RPL + r] = S[r];
   }
 }
 
 // q, k [T, kv_heads * dim] and v [T, heads * vdim] of the run's type with their row strides; ab float32 [T, 2 heads]
-// (a then b); a_log, dt_bias float32 [heads]; state: slot s at state + s * state_stride, [heads, dim, vdim];
+// (a then b); a_log, dt_bias float32 [heads]; state: slot s at state + s * state_stride, [heads, vdim, dim] (a column's rows side by side);
 // out float32 [T, heads, vdim].
 extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dtype, int64_t q_stride,
                              int64_t k_stride, int64_t v_stride, const float* ab, const float* a_log,
@@ -338,7 +362,8 @@ extern "C" int ix_delta_rule(const void* q, const void* k, const void* v, int dt
   // 16-byte pieces: a lane's quarter of a head is a multiple of eight numbers, and rows and heads start aligned
   const int elt = 2;
   const bool vec = dtype == IX_BF16 && dim % (8 * DELTA_SPLIT) == 0 && (q_stride * elt) % 16 == 0 && (k_stride * elt) % 16 == 0 &&
-                   ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k)) & 15) == 0;
+                   state_stride % 4 == 0 &&
+                   ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(state)) & 15) == 0;
 #define LAUNCH(TT, RPL, VEC)                                                                                            \
   hipLaunchKernelGGL((delta_rule_kernel<TT, RPL, VEC>), grid, block, 0, stream, (const TT*)q, (const TT*)k, (const TT*)v, \
                      q_stride, k_stride, v_stride, ab, a_log, dt_bias, state, state_stride, q_start, state_slots, out,    \

@@ -7,7 +7,7 @@
     S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q                        S [dim, vdim] float32
     y          = (o / rms(o) * norm_weight * silu(gate)) . Wo^T                         rms over a head's vdim
 
-Query head h reads the q/k head h / (heads / kv_heads).  State per request: the heads' matrices and the short
+Query head h reads the q/k head h / (heads / kv_heads).  State per request: the heads' matrices (a column's rows side by side, as the kernels read them) and the short
 convolution's last inputs, both float32, in the request's state slot; nothing is kept in pages.  Decays, step
 sizes, unit norms, the recurrence and the head norm are float32 in every run.
 """

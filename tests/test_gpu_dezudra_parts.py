@@ -233,7 +233,7 @@ def plain_delta(q, k, v, a, b, a_log, dt_bias, heads, kv_heads, dim, vdim):
 
 
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim", [(4, 2, 32, 48), (3, 1, 20, 12), (1, 1, 128, 16), (2, 2, 7, 70),
-                                                     (2, 1, 200, 17)])
+                                                     (2, 1, 200, 17), (2, 1, 64, 40), (1, 1, 96, 32), (2, 2, 128, 20)])
 @pytest.mark.parametrize("dtype,tol", TYPES)
 def test_delta_rule_over_steps(dtype, tol, heads, kv_heads, dim, vdim):
     from inferx_amd import ops
@@ -242,7 +242,8 @@ def test_delta_rule_over_steps(dtype, tol, heads, kv_heads, dim, vdim):
     vs = [rnd((n, heads * vdim), 50 + r, 1.0, dtype) for r, n in enumerate(LENGTHS)]
     abs_ = [rnd((n, 2 * heads), 60 + r, 1.5) for r, n in enumerate(LENGTHS)]
     a_log, dt_bias = rnd((heads,), 5, 0.7), rnd((heads,), 6, 0.7)
-    state = torch.full((2, heads * dim * vdim + 11), float("nan"), device=DEV)
+    # (blocks of a multiple of four numbers let the kernel read the state in 16-byte pieces: both ways are run)
+    state = torch.full((2, heads * dim * vdim + (12 if vdim % 16 == 0 else 11)), float("nan"), device=DEV)
     want = {r: plain_delta(f64(qs[r]), f64(ks[r]), f64(vs[r]), f64(abs_[r])[:, :heads], f64(abs_[r])[:, heads:],
                            f64(a_log), f64(dt_bias), heads, kv_heads, dim, vdim) for r in range(3)}
 
