@@ -9,10 +9,12 @@
 //
 // The columns of S are independent recurrences (column j only ever meets v[j]), so the work is spread over
 // (request, head, block of 16 value columns): one wavefront each, four lanes per column that own every fourth row
-// of it (RPL rows a lane, in registers; VEC: a quarter of the rows each, side by side, where that quarter is a multiple
-// of eight numbers and 16-byte aligned, so that a lane reads its part of q and k in 16-byte pieces).  A wavefront walks its request's rows of this step in order, with the
-// next row's operands asked for before the present row is worked; the state is read from the request's slot at the
-// start and written back at the end.  Query head h reads the q/k head h / (heads / kv_heads).
+// of it (RPL rows a lane, in registers; VEC: a quarter of the rows each, side by side, where that quarter is a
+// multiple of eight numbers and everything is 16-byte aligned, so that a lane reads its part of q and k, and of
+// the state, in 16-byte pieces).  A wavefront walks its request's rows of this step in order, with the next row's
+// operands asked for before the present row is worked; the state is read from the request's slot at the start and
+// written back at the end.  In the slot a head's matrix lies [column][row], a column's rows side by side.
+// Query head h reads the q/k head h / (heads / kv_heads).
 #include "common.h"
 
 typedef unsigned int delta_u32x4 __attribute__((ext_vector_type(4)));

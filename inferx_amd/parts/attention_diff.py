@@ -83,7 +83,7 @@ class DifferentialAttention(Mixer):
         self.w_qkv = stack_rows([tensors[f"{n}.weight"] for n in "qkv"])
         self.b_qkv = stack_rows([tensors[f"{n}.bias"] for n in "qkv"])
         self.w_out = tensors["o.weight"].contiguous()
-        self.conv.bind(tensors)
+        self.conv.bind(tensors, bias=self.b_qkv)
         dot = lambda a, b: float((tensors[a].double() * tensors[b].double()).sum().item())
         self.lam = math.exp(dot("lq1", "lk1")) - math.exp(dot("lq2", "lk2")) + self.diff
         if self.position is not None:
@@ -95,11 +95,10 @@ class DifferentialAttention(Mixer):
         proj = rt.linear(x, self.w_qkv)
         q = rt.empty((T, self.num_heads, 2, self.head_dim))
         if cache.writes:
-            self.conv.apply(ctx, proj, self.b_qkv, cache.state, q, cache.k, cache.v, slots=ctx.slots[cache.group],
-                            cos_sin=table)
+            self.conv.apply(ctx, proj, cache.state, q, cache.k, cache.v, slots=ctx.slots[cache.group], cos_sin=table)
         else:  # the keys and values are another execution's: only the queries are wanted
-            self.conv.apply(ctx, proj, self.b_qkv, cache.state, q, rt.empty((T, self.k_dim)),
-                            rt.empty((T, self.v_dim)), cos_sin=table)
+            self.conv.apply(ctx, proj, cache.state, q, rt.empty((T, self.k_dim)), rt.empty((T, self.v_dim)),
+                            cos_sin=table)
         out = rt.empty((T, self.num_heads, self.value_dim))
         self.attend(ctx, q, cache, out)
         return rt.linear(out.view(T, self.o_dim), self.w_out)

@@ -67,7 +67,7 @@ class GatedDeltaMixer(Mixer):
         ab = rt.linear_f32(x, self.w_ab)      # the decay's and the step size's logits, float32
         q, k, v = rt.empty((T, self.qk_dim)), rt.empty((T, self.qk_dim)), rt.empty((T, self.v_dim))
         matrices, tail = cache.state[:, :self.matrix_floats], cache.state[:, self.matrix_floats:]
-        self.conv.apply(ctx, proj, None, tail, q, k, v, silu=True)
+        self.conv.apply(ctx, proj, tail, q, k, v, silu=True)
         o = rt.empty((T, self.num_heads, self.value_dim), torch.float32)
         ops.delta_rule(q, k, v, ab, self.a_log, self.dt_bias, matrices,
                        ops.StepRows(ctx.seq_of_token, ctx.q_start, ctx.state_slots), o, self.num_heads,

@@ -25,8 +25,7 @@ class ShortConv:
         self.sizes: Tuple[int, int, int, int, int] = (int(q_channels), int(k_channels), int(v_channels),
                                                       int(head_dim), int(value_dim))
         self.taps = int(taps)
-        self.weight = self.weight_t = None
-        self._bias_f32 = (None, None)  # (the bias it was made from, its float32 copy)
+        self.weight = self.weight_t = self.bias = self.bias_f32 = None
 
     @property
     def channels(self) -> int:
@@ -40,15 +39,15 @@ class ShortConv:
         """One [channels, taps] tensor per run of channels, named `<name>.conv`."""
         return [ParamSpec(f"{n}.conv", (c, self.taps), std=std) for n, c in zip(names, self.sizes[:3])]
 
-    def bind(self, tensors, names=("q", "k", "v")) -> None:
+    def bind(self, tensors, names=("q", "k", "v"), bias=None) -> None:
+        """`bias`: what is added to the inputs before the convolution (one number per channel), or None."""
+        self.bias = bias
+        self.bias_f32 = bias.to(torch.float32).contiguous() if bias is not None else None
         self.weight = stack_rows([tensors[f"{n}.conv"] for n in names])
         self.weight_t = self.weight.to(torch.float32).t().contiguous()  # [taps, channels], for the kernel's 16-byte form
 
-    def apply(self, ctx, x, bias, state, out_q, out_k, out_v, slots=None, cos_sin=None, silu: bool = False) -> None:
+    def apply(self, ctx, x, state, out_q, out_k, out_v, slots=None, cos_sin=None, silu: bool = False) -> None:
         """`state`: the float32 view [slots, >= state_floats] of the requests' last inputs (see `ops.short_conv`)."""
         rows = ops.StepRows(ctx.seq_of_token, ctx.q_start, ctx.state_slots)
-        if bias is not None and self._bias_f32[0] is not bias:
-            self._bias_f32 = (bias, bias.to(torch.float32).contiguous())
-        ops.short_conv(x, bias, self.weight, state, rows, self.sizes, out_q, out_k, out_v, slots=slots,
-                       cos_sin=cos_sin, silu=silu, weight_t=self.weight_t,
-                       bias_f32=self._bias_f32[1] if bias is not None else None)
+        ops.short_conv(x, self.bias, self.weight, state, rows, self.sizes, out_q, out_k, out_v, slots=slots,
+                       cos_sin=cos_sin, silu=silu, weight_t=self.weight_t, bias_f32=self.bias_f32)

@@ -553,3 +553,43 @@ def test_one_key_stands_out_at_every_edge_on_the_matrix_cores(grouped):
                 err = float(np.abs(f64(out)[0, 0] - target).max())
                 assert np.isfinite(f64(out)).all(), f"query {pos}, key {key}: not-a-number read"
                 assert (err < 3e-2) == seen, f"query {pos}, key {key}, {n_splits} slices: {'not ' if seen else ''}found (error {err:.2e})"
+
+
+@pytest.mark.parametrize("kernel", ["plain", "matrix cores", "matrix cores, 4 slices"])
+def test_one_key_stands_out_for_every_query_of_a_portion(kernel):
+    """A prompt portion of 48 queries that all point at ONE key: every query finds it exactly if it sees it (at or
+    before its own position, and within its own window or among the kept first tokens), whatever its place in its
+    tile of 16; the portion ends at a page's edge, in the middle of a page, and right after the window has filled."""
+    from inferx_amd import ops
+    H, G, D, V, L, page = 2, 1, 16, 32, 400, 16
+    window, keep = 37, 5
+    dtype = torch.bfloat16
+    k = rnd((L, 2 * G, D), 1, 0.05)
+    v = rnd((L, G, V), 2, 1.0)
+    mark = torch.zeros(D)
+    mark[7] = 1.0
+    eps = 1e-6
+    for last in (47, 63, 100, 255, 399):
+        positions = list(range(last - 47, last + 1))
+        for key in (0, keep - 1, keep, last - 47 - window, last - 47 - window + 1, last - window, last - window + 1,
+                    last - 60, last - 47, last - 20, last - 16, last - 15, last):
+            if key < 0:
+                continue
+            kk = k.clone()
+            kk[key, 0] = mark * 40.0
+            q = torch.zeros((48, H, 2, D))
+            q[:, :, 0] = mark * 40.0
+            kc, vc, table = paged(kk.to(dtype), v.to(dtype), page, dtype, seed=last)
+            if kernel == "plain":
+                out = torch.empty((48, H, V), dtype=dtype, device=DEV)
+                ops.attention_diff_plain(q.to(dtype).to(DEV), kc, vc, table, i32([0] * 48), i32(positions), out, 1.0, window,
+                                         keep, 0.0, eps, 1.0)
+            else:
+                out = mfma_attend(q.to(dtype), kc, vc, table, tiles_of([(0, 0, 48)]), positions, 4 if "slices" in kernel else 1,
+                                  1.0, window, keep, 0.0, eps, 1.0)
+            target = f64(v.to(dtype))[key, 0]
+            target = target / np.sqrt(np.mean(target * target) + eps)
+            err = np.abs(f64(out)[:, 0] - target[None, :]).max(axis=1)
+            seen = np.array([key <= p and (p - key < window or key < keep) for p in positions])
+            assert np.array_equal(err < 3e-2, seen), \
+                f"portion ending at {last}, key {key}: queries {np.flatnonzero((err < 3e-2) != seen).tolist()} of the portion are wrong"
